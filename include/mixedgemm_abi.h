@@ -1,0 +1,108 @@
+/*
+ * C-ABI of the MI355X (gfx950) reorder-quantize + mixed MXFP4/6/8 GEMM library.
+ *
+ * Plain C types only: device pointers, sizes, a HIP stream passed as void*.
+ * Every entry point validates its arguments on the host, enqueues its kernels
+ * on `stream` and returns without synchronizing; none allocates.  The return
+ * value is a status code: 0 on success, a hipError_t value for a HIP failure, or
+ * one of the MG_ERR_* codes below.  mg_status_string() names any of them.
+ *
+ * Citations give the reference interface each entry point replaces, relative
+ * to the reference tree.
+ */
+#ifndef MIXEDGEMM_ABI_H
+#define MIXEDGEMM_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MG_OK 0
+#define MG_ERR_BAD_SHAPE 10001   /* a segment is not a multiple of 32, K mismatch, negative size */
+#define MG_ERR_BAD_POINTER 10002 /* null or insufficiently aligned pointer (16 bytes required) */
+#define MG_ERR_BAD_INDEX 10003   /* reorder index entry outside [0, K) (only when checked on host) */
+#define MG_ERR_UNSUPPORTED 10004 /* shape outside what the kernels handle (K > 32736) */
+
+/* Operand selector for mg_sf_bytes(). */
+#define MG_OPERAND_A 0 /* activations: (rows/128 + 1)*128*kseg/32, src/bindings.cpp:91-93 */
+#define MG_OPERAND_B 1 /* weights:     rows*kseg/32,               src/bindings.cpp:210-212 */
+
+/*
+ * Activation reorder-quantize.  Replaces run_reorder_bf16_mixed<32,K>
+ * (include/reorder.cuh:295-308, src/reorder.cu:434-469) and its kernel
+ * reorder_bf16_mixed_kernel (src/reorder.cu:94-269), for any K that is a
+ * multiple of 32 (the reference instantiates seven values of K only).
+ *
+ *   x_bf16 [M, K] bf16 row-major, idx [K] int16 (output position j takes input
+ *   channel idx[j]); K = KN + KS + KO, each a multiple of 32.
+ *   qn [M, KN/2]   E2M1 codes, element 2i in the low nibble of byte i
+ *   qs [M, 3KS/4]  E3M2 codes, 4 codes per 3 bytes, little-endian bit stream
+ *   qo [M, KO]     E4M3 codes
+ *   sfn/sfs/sfo    E8M0 scale bytes, one per 32 elements, in the 128-row x
+ *                  4-block interleaved layout; mg_sf_bytes(M, Kseg, MG_OPERAND_A)
+ *                  bytes each.  Entries of rows >= M are left untouched.
+ */
+int mg_reorder_quantize_x(const void* x_bf16, const int16_t* idx, int M, int K, int KN, int KS, int KO,
+                          uint8_t* qn, uint8_t* qs, uint8_t* qo,
+                          uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream);
+
+/*
+ * Weight reorder-quantize: same gather and scale rule, all three segments to
+ * E2M1.  Replaces run_reorder_bf16_fp4<32,K> (include/reorder.cuh:310-323,
+ * src/reorder.cu:471-506) and reorder_bf16_fp4_kernel (src/reorder.cu:271-432).
+ *   qn [N, KN/2], qs [N, KS/2], qo [N, KO/2]; scale buffers of
+ *   mg_sf_bytes(N, Kseg, MG_OPERAND_B) bytes.
+ */
+int mg_reorder_quantize_w(const void* w_bf16, const int16_t* idx, int N, int K, int KN, int KS, int KO,
+                          uint8_t* qn, uint8_t* qs, uint8_t* qo,
+                          uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream);
+
+/*
+ * Mixed block-scaled GEMM: D[M,N] = bf16( sum over the three K segments of
+ * A_seg . B_seg^T ), fp32 accumulation across all segments, one bf16 rounding.
+ * Replaces matmul_host (include/gemm.h:21-41, src/gemm.cu:22-47) and the three
+ * segment GEMMs it chains (src/fp4.cu:35, src/fp6.cu:35, src/fp8.cu:35).
+ * Operand layouts are the ones the two quantizers above produce.
+ */
+int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
+                  const uint8_t* ao, const uint8_t* bo,
+                  const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
+                  const uint8_t* sfao, const uint8_t* sfbo,
+                  int M, int N, int KN, int KS, int KO, void* d_bf16, void* stream);
+
+/*
+ * Activation reorder-quantize followed by the mixed GEMM on the same stream
+ * (the sequence src/bindings.cpp:69-186 then :9-67 performs with a device-wide
+ * synchronize in between; bench_reorder_gemm.cu:163-167 times the same pair).
+ * `workspace` receives the quantized activations and their scales;
+ * mg_fused_workspace_bytes(M, KN, KS, KO) bytes, 256-byte aligned.
+ */
+int mg_fused_linear(const void* x_bf16, const int16_t* idx,
+                    const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                    const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo,
+                    int M, int N, int KN, int KS, int KO,
+                    void* d_bf16, void* workspace, size_t workspace_bytes, void* stream);
+size_t mg_fused_workspace_bytes(int M, int KN, int KS, int KO);
+
+/* Size in bytes of one segment's scale buffer (src/bindings.cpp:91-93, 210-212);
+ * never smaller than the interleaved layout spans. */
+size_t mg_sf_bytes(int rows, int kseg, int operand);
+
+/* Byte offset of the scale of (row, 32-element block kb) inside a segment's
+ * scale buffer (include/reorder.cuh:119-124; src/reorder.cu:182-185). */
+size_t mg_sf_offset(int row, int kb, int kseg);
+
+/* Blocks the host until all work on the current device has finished
+ * (src/bindings.cpp:59,178,297 do this after every operator). */
+int mg_device_synchronize(void);
+
+/* Text for a status code returned by any function above. */
+const char* mg_status_string(int status);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MIXEDGEMM_ABI_H */

@@ -1,0 +1,158 @@
+"""ctypes binding of the C-ABI in include/mixedgemm_abi.h.
+
+Device memory and streams come from torch; every compute call goes into
+libmixedgemm_hip.so.  There is no fallback: if the library has not been built
+the first call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libmixedgemm_hip.so")
+
+MG_OPERAND_A = 0
+MG_OPERAND_B = 1
+
+SYMBOLS = (
+    "mg_reorder_quantize_x", "mg_reorder_quantize_w", "mg_mixed_gemm", "mg_fused_linear",
+    "mg_fused_workspace_bytes", "mg_sf_bytes", "mg_sf_offset", "mg_device_synchronize", "mg_status_string",
+)
+
+_lib = None
+
+
+class MixedGemmError(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise MixedGemmError(
+                f"{LIB_PATH} is missing: build it with `python -m mixedgemm_amd.build` "
+                "(there is no non-HIP fallback)")
+        L = ctypes.CDLL(LIB_PATH)
+        p, i, z = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+        for name in ("mg_reorder_quantize_x", "mg_reorder_quantize_w"):
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = i, [p, p, i, i, i, i, i, p, p, p, p, p, p, p]
+        L.mg_mixed_gemm.restype, L.mg_mixed_gemm.argtypes = i, [p] * 12 + [i] * 5 + [p, p]
+        L.mg_fused_linear.restype = i
+        L.mg_fused_linear.argtypes = [p] * 8 + [i] * 5 + [p, p, z, p]
+        L.mg_fused_workspace_bytes.restype, L.mg_fused_workspace_bytes.argtypes = z, [i, i, i, i]
+        L.mg_sf_bytes.restype, L.mg_sf_bytes.argtypes = z, [i, i, i]
+        L.mg_sf_offset.restype, L.mg_sf_offset.argtypes = z, [i, i, i]
+        L.mg_device_synchronize.restype, L.mg_device_synchronize.argtypes = i, []
+        L.mg_status_string.restype, L.mg_status_string.argtypes = ctypes.c_char_p, [i]
+        _lib = L
+    return _lib
+
+
+def status_string(status: int) -> str:
+    return lib().mg_status_string(int(status)).decode()
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        raise MixedGemmError(f"{what} failed: {status_string(status)} (status {status})")
+
+
+def sf_bytes(rows: int, kseg: int, operand: int) -> int:
+    return int(lib().mg_sf_bytes(rows, kseg, operand))
+
+
+def sf_offset(row: int, kb: int, kseg: int) -> int:
+    return int(lib().mg_sf_offset(row, kb, kseg))
+
+
+def fused_workspace_bytes(m: int, kn: int, ks: int, ko: int) -> int:
+    return int(lib().mg_fused_workspace_bytes(m, kn, ks, ko))
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() else ctypes.c_void_p(0)
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
+    if t.dtype != dtype:
+        raise MixedGemmError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_cuda:
+        raise MixedGemmError(f"{name}: expected a GPU tensor")
+    if not t.is_contiguous():
+        raise MixedGemmError(f"{name}: expected a contiguous tensor")
+
+
+def _reorder_quantize(fn_name, operand, t, idx, kn, ks, ko):
+    _require(t, torch.bfloat16, "input")
+    _require(idx, torch.int16, "reorder_index")
+    rows, k = t.shape
+    if idx.numel() != k:
+        raise MixedGemmError(f"reorder_index has {idx.numel()} entries, input has {k} channels")
+    w = operand == MG_OPERAND_B
+    u8 = dict(dtype=torch.uint8, device=t.device)
+    qn = torch.empty((rows, kn // 2), **u8)
+    qs = torch.empty((rows, ks // 2 if w else ks // 4 * 3), **u8)
+    qo = torch.empty((rows, ko // 2 if w else ko), **u8)
+    sfn = torch.empty(sf_bytes(rows, kn, operand), **u8)
+    sfs = torch.empty(sf_bytes(rows, ks, operand), **u8)
+    sfo = torch.empty(sf_bytes(rows, ko, operand), **u8)
+    status = getattr(lib(), fn_name)(_ptr(t), _ptr(idx), rows, k, kn, ks, ko,
+                                     _ptr(qn), _ptr(qs), _ptr(qo), _ptr(sfn), _ptr(sfs), _ptr(sfo), _stream(t))
+    check(status, fn_name)
+    return qn, qs, qo, sfn, sfs, sfo
+
+
+def reorder_quantize_x(x, reorder_index, kn, ks, ko):
+    """(XN, XS, XO, SFXN, SFXS, SFXO); asynchronous on torch's current stream."""
+    return _reorder_quantize("mg_reorder_quantize_x", MG_OPERAND_A, x, reorder_index, kn, ks, ko)
+
+
+def reorder_quantize_w(w, reorder_index, kn, ks, ko):
+    """(WN, WS, WO, SFWN, SFWS, SFWO); asynchronous on torch's current stream."""
+    return _reorder_quantize("mg_reorder_quantize_w", MG_OPERAND_B, w, reorder_index, kn, ks, ko)
+
+
+def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None):
+    """bf16 [M, N]; shapes are recovered from the packed operands."""
+    for name, t in (("AN", an), ("BN", bn), ("AS", as_), ("BS", bs), ("AO", ao), ("BO", bo),
+                    ("SFAN", sfan), ("SFBN", sfbn), ("SFAS", sfas), ("SFBS", sfbs), ("SFAO", sfao), ("SFBO", sfbo)):
+        _require(t, torch.uint8, name)
+    m, n = an.shape[0], bn.shape[0]
+    kn, ks, ko = an.shape[1] * 2, as_.shape[1] * 4 // 3, ao.shape[1]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=an.device)
+    status = lib().mg_mixed_gemm(_ptr(an), _ptr(bn), _ptr(as_), _ptr(bs), _ptr(ao), _ptr(bo),
+                                 _ptr(sfan), _ptr(sfbn), _ptr(sfas), _ptr(sfbs), _ptr(sfao), _ptr(sfbo),
+                                 m, n, kn, ks, ko, _ptr(out), _stream(an))
+    check(status, "mg_mixed_gemm")
+    return out
+
+
+def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, workspace=None, out=None):
+    """Activation reorder-quantize + mixed GEMM on one stream; returns bf16 [M, N]."""
+    _require(x, torch.bfloat16, "X")
+    _require(reorder_index, torch.int16, "reorder_index")
+    m, n = x.shape[0], bn.shape[0]
+    need = fused_workspace_bytes(m, kn, ks, ko)
+    if workspace is None:
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    status = lib().mg_fused_linear(_ptr(x), _ptr(reorder_index), _ptr(bn), _ptr(bs), _ptr(bo),
+                                   _ptr(sfbn), _ptr(sfbs), _ptr(sfbo), m, n, kn, ks, ko,
+                                   _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
+    check(status, "mg_fused_linear")
+    return out
+
+
+def device_synchronize() -> None:
+    check(lib().mg_device_synchronize(), "mg_device_synchronize")

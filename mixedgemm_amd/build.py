@@ -1,0 +1,89 @@
+"""Builds the HIP library (C-ABI) and the pybind11/torch extension module.
+
+    python -m mixedgemm_amd.build            # build what is missing or stale
+    python -m mixedgemm_amd.build --force    # rebuild everything
+
+Outputs (kept out of git, shipped with the tree):
+    mixedgemm_amd/lib/libmixedgemm_hip.so   hand-written gfx950 kernels + extern "C" entry points
+    build/mixedgemm.so                      torch extension with the reference's operator surface
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+import sysconfig
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIB_DIR = os.path.join(PKG, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libmixedgemm_hip.so")
+EXT_DIR = os.path.join(ROOT, "build")
+EXT_PATH = os.path.join(EXT_DIR, "mixedgemm.so")
+
+HIP_SOURCES = ["abi.hip", "reorder_quant.hip", "mixed_gemm.hip"]
+HIP_HEADERS = ["mg_common.h", os.path.join(ROOT, "include", "mixedgemm_abi.h")]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed FP32 VALU forms are kept out of every kernel
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _stale(target: str, deps: list[str]) -> bool:
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build_hip_library(force: bool = False, verbose: bool = False) -> str:
+    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
+    deps = srcs + [h if os.path.isabs(h) else os.path.join(CSRC, h) for h in HIP_HEADERS]
+    if force or _stale(LIB_PATH, deps):
+        os.makedirs(LIB_DIR, exist_ok=True)
+        cmd = ["hipcc", *HIPCC_FLAGS, "-o", LIB_PATH, *srcs]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+def build_torch_extension(force: bool = False, verbose: bool = False) -> str:
+    """g++ build of csrc/bindings.cpp against torch + pybind11; links the HIP
+    library through its C-ABI only (no HIP headers on this side)."""
+    import torch
+    from torch.utils import cpp_extension
+
+    src = os.path.join(CSRC, "bindings.cpp")
+    deps = [src, os.path.join(ROOT, "include", "mixedgemm_abi.h"), LIB_PATH]
+    if force or _stale(EXT_PATH, deps):
+        os.makedirs(EXT_DIR, exist_ok=True)
+        torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+        inc = [f"-I{p}" for p in cpp_extension.include_paths()]
+        inc += [f"-I{sysconfig.get_paths()['include']}", f"-I{os.path.join(ROOT, 'include')}"]
+        cmd = [
+            "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+            "-DTORCH_EXTENSION_NAME=mixedgemm", "-DTORCH_API_INCLUDE_EXTENSION_H",
+            "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-I/opt/rocm/include",
+            f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+            *inc, src, "-o", EXT_PATH,
+            f"-L{LIB_DIR}", "-lmixedgemm_hip", f"-Wl,-rpath,{LIB_DIR}", "-Wl,-rpath,$ORIGIN/../mixedgemm_amd/lib",
+            f"-L{torch_lib}", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_python", f"-Wl,-rpath,{torch_lib}",
+        ]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+    return EXT_PATH
+
+
+def build_all(force: bool = False, verbose: bool = False) -> None:
+    build_hip_library(force, verbose)
+    build_torch_extension(force, verbose)
+
+
+if __name__ == "__main__":
+    build_all(force="--force" in sys.argv, verbose=True)

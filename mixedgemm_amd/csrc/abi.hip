@@ -1,0 +1,127 @@
+// extern "C" surface of the library: argument validation on the host, then the
+// kernel launchers.  Nothing here allocates or synchronizes (except
+// mg_device_synchronize, whose only job that is).
+#include "../../include/mixedgemm_abi.h"
+
+#include "mg_common.h"
+
+namespace mg {
+template <bool IS_W>
+hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int K, int KN, int KS, int KO, uint8_t* qn,
+                                uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, hipStream_t stream);
+hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
+                             const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
+                             const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
+                             int N, int KN, int KS, int KO, void* d, hipStream_t stream);
+}  // namespace mg
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// A segment pointer may be null only when that segment is empty.
+bool ptr_ok(const void* p, bool needed) { return needed ? (p != nullptr && aligned16(p)) : true; }
+
+int check_split(int rows, int KN, int KS, int KO) {
+  if (rows < 0 || KN < 0 || KS < 0 || KO < 0) return MG_ERR_BAD_SHAPE;
+  if ((KN | KS | KO) & 31) return MG_ERR_BAD_SHAPE;
+  if ((long long)KN + KS + KO > 32736) return MG_ERR_UNSUPPORTED;  // int16 index, one lane per block, <= 1024 lanes
+  return MG_OK;
+}
+
+template <bool IS_W>
+int reorder_quantize(const void* x, const int16_t* idx, int rows, int K, int KN, int KS, int KO, uint8_t* qn,
+                     uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream) {
+  if (int s = check_split(rows, KN, KS, KO)) return s;
+  if (K != KN + KS + KO) return MG_ERR_BAD_SHAPE;
+  if (rows == 0 || K == 0) return MG_OK;
+  if (!ptr_ok(x, true) || !ptr_ok(idx, true)) return MG_ERR_BAD_POINTER;
+  if (!ptr_ok(qn, KN > 0) || !ptr_ok(qs, KS > 0) || !ptr_ok(qo, KO > 0)) return MG_ERR_BAD_POINTER;
+  if ((KN > 0 && !sfn) || (KS > 0 && !sfs) || (KO > 0 && !sfo)) return MG_ERR_BAD_POINTER;
+  return (int)mg::launch_reorder_quant<IS_W>(x, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo,
+                                             static_cast<hipStream_t>(stream));
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+}  // namespace
+
+extern "C" {
+
+int mg_reorder_quantize_x(const void* x_bf16, const int16_t* idx, int M, int K, int KN, int KS, int KO, uint8_t* qn,
+                          uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream) {
+  return reorder_quantize<false>(x_bf16, idx, M, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream);
+}
+
+int mg_reorder_quantize_w(const void* w_bf16, const int16_t* idx, int N, int K, int KN, int KS, int KO, uint8_t* qn,
+                          uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream) {
+  return reorder_quantize<true>(w_bf16, idx, N, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream);
+}
+
+int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs, const uint8_t* ao,
+                  const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
+                  const uint8_t* sfao, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO, void* d_bf16,
+                  void* stream) {
+  if (int s = check_split(M, KN, KS, KO)) return s;
+  if (N < 0) return MG_ERR_BAD_SHAPE;
+  if (M == 0 || N == 0) return MG_OK;
+  if (!ptr_ok(d_bf16, true)) return MG_ERR_BAD_POINTER;
+  if (!ptr_ok(an, KN > 0) || !ptr_ok(bn, KN > 0) || !ptr_ok(as_, KS > 0) || !ptr_ok(bs, KS > 0) ||
+      !ptr_ok(ao, KO > 0) || !ptr_ok(bo, KO > 0))
+    return MG_ERR_BAD_POINTER;
+  if ((KN > 0 && (!sfan || !sfbn)) || (KS > 0 && (!sfas || !sfbs)) || (KO > 0 && (!sfao || !sfbo)))
+    return MG_ERR_BAD_POINTER;
+  return (int)mg::launch_mixed_gemm(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, N, KN, KS, KO, d_bf16,
+                                    static_cast<hipStream_t>(stream));
+}
+
+size_t mg_sf_bytes(int rows, int kseg, int operand) {
+  if (rows < 0 || kseg < 0) return 0;
+  const size_t span = (size_t)((rows + 127) / 128) * (size_t)((kseg + 127) / 128) * 512;
+  const size_t ref = operand == MG_OPERAND_A ? (size_t)(rows / 128 + 1) * 128 * (size_t)kseg / 32
+                                             : (size_t)rows * (size_t)kseg / 32;
+  return ref > span ? ref : span;
+}
+
+size_t mg_sf_offset(int row, int kb, int kseg) { return mg::sf_offset(row, kb, (kseg + 127) / 128); }
+
+size_t mg_fused_workspace_bytes(int M, int KN, int KS, int KO) {
+  if (M < 0 || KN < 0 || KS < 0 || KO < 0) return 0;
+  return align256((size_t)M * (KN / 2)) + align256((size_t)M * (KS / 4 * 3)) + align256((size_t)M * KO) +
+         align256(mg_sf_bytes(M, KN, MG_OPERAND_A)) + align256(mg_sf_bytes(M, KS, MG_OPERAND_A)) +
+         align256(mg_sf_bytes(M, KO, MG_OPERAND_A));
+}
+
+int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                    const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO,
+                    void* d_bf16, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int s = check_split(M, KN, KS, KO)) return s;
+  if (N < 0) return MG_ERR_BAD_SHAPE;
+  if (M == 0 || N == 0) return MG_OK;
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return MG_ERR_BAD_POINTER;
+  if (workspace_bytes < mg_fused_workspace_bytes(M, KN, KS, KO)) return MG_ERR_BAD_SHAPE;
+  uint8_t* p = static_cast<uint8_t*>(workspace);
+  uint8_t* qn = p;  p += align256((size_t)M * (KN / 2));
+  uint8_t* qs = p;  p += align256((size_t)M * (KS / 4 * 3));
+  uint8_t* qo = p;  p += align256((size_t)M * KO);
+  uint8_t* sfn = p; p += align256(mg_sf_bytes(M, KN, MG_OPERAND_A));
+  uint8_t* sfs = p; p += align256(mg_sf_bytes(M, KS, MG_OPERAND_A));
+  uint8_t* sfo = p;
+  if (int s = mg_reorder_quantize_x(x_bf16, idx, M, KN + KS + KO, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream)) return s;
+  return mg_mixed_gemm(qn, bn, qs, bs, qo, bo, sfn, sfbn, sfs, sfbs, sfo, sfbo, M, N, KN, KS, KO, d_bf16, stream);
+}
+
+int mg_device_synchronize(void) { return (int)hipDeviceSynchronize(); }
+
+const char* mg_status_string(int status) {
+  switch (status) {
+    case MG_OK: return "success";
+    case MG_ERR_BAD_SHAPE: return "invalid shape: segment sizes must be non-negative multiples of 32 and K = KN + KS + KO";
+    case MG_ERR_BAD_POINTER: return "null or misaligned pointer (16-byte alignment required)";
+    case MG_ERR_BAD_INDEX: return "reorder index entry out of range";
+    case MG_ERR_UNSUPPORTED: return "unsupported shape: K must not exceed 32736";
+    default: return hipGetErrorString(static_cast<hipError_t>(status));
+  }
+}
+
+}  // extern "C"

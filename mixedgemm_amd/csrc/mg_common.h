@@ -1,0 +1,36 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mg {
+
+constexpr int kGroup = 32;  // elements per shared scale (src/reorder.cu:78-79 of the reference)
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned v6u __attribute__((ext_vector_type(6)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef __bf16 v32bf __attribute__((ext_vector_type(32)));
+typedef short v2s __attribute__((ext_vector_type(2)));
+
+// MFMA f8f6f4 operand format selectors (cbsz for operand A, blgp for operand B).
+constexpr int kFmtE4M3 = 0;
+constexpr int kFmtE3M2 = 3;
+constexpr int kFmtE2M1 = 4;
+
+// Byte offset of the scale of (row r, block kb) in a segment's scale buffer:
+// 128-row x 4-block atoms of 512 bytes, atoms along K fastest
+// (include/reorder.cuh:119-124, src/reorder.cu:182-185 of the reference).
+__host__ __device__ inline size_t sf_offset(int r, int kb, int katoms) {
+  return ((size_t)(r >> 7) * katoms + (kb >> 2)) * 512 + (r & 31) * 16 + ((r >> 5) & 3) * 4 + (kb & 3);
+}
+
+__host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+}  // namespace mg

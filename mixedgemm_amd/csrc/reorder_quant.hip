@@ -1,0 +1,248 @@
+// Reorder-quantize kernels for gfx950: gather bf16 channels by a reorder index,
+// then per-32-element power-of-two (E8M0) scaling and quantization into packed
+// MXFP4 (E2M1) / MXFP6 (E3M2) / MXFP8 (E4M3) segments.
+//
+// Semantics follow the reference kernels reorder_bf16_mixed_kernel
+// (src/reorder.cu:94-269) and reorder_bf16_fp4_kernel (src/reorder.cu:271-432):
+//   scale  = 2^e, e = min{e : amax <= MAX * 2^e}  (= ceil(log2(amax/MAX)), :180),
+//            0.5 for an all-zero block (:179); E8M0 byte = e + 127
+//   code   = RNE_fmt( bf16( clamp( roundf(x / scale) ) ) )   (:221-248)
+// The design is not the reference's: a workgroup stages R rows at a time into
+// LDS in channel-major order with the R rows of one channel adjacent, so one
+// 2R-byte LDS read fetches a gathered channel for all R rows; one lane owns one
+// 32-element block (no cross-lane reduction), the scale exponent comes from
+// integer arithmetic on the float bits, and the element conversion is done by
+// the gfx950 cvt_scalef32 instructions on the already integer-rounded values.
+#include "mg_common.h"
+
+namespace mg {
+
+namespace {
+
+__device__ __forceinline__ unsigned perm(unsigned hi, unsigned lo, unsigned sel) {
+  return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+// E8M0 byte of the block scale from the bits of amax (a non-negative float).
+// MAX = fm * 2^pm with fm in [0.5,1): the exponent steps up by one when the
+// mantissa of amax exceeds the mantissa of MAX, which the add below carries
+// into the exponent field.
+template <int FMT>
+__device__ __forceinline__ int scale_byte(float amax) {
+  constexpr unsigned thr = (FMT == kFmtE2M1) ? 0x400000u : 0x600000u;  // 6 = 1.5*4, 28 = 1.75*16, 448 = 1.75*256
+  constexpr int pm = (FMT == kFmtE2M1) ? 3 : (FMT == kFmtE3M2 ? 5 : 9);
+  unsigned bits = __float_as_uint(amax);
+  int byte = (int)((bits + (0x7FFFFFu - thr)) >> 23) + 1 - pm;
+  byte = byte < 0 ? 0 : byte;
+  return amax == 0.0f ? 126 : byte;
+}
+
+// roundf(x * rs): half away from zero, sign of zero kept.
+__device__ __forceinline__ float round_scaled(float x, float rs) {
+  float half = __uint_as_float((__float_as_uint(x) & 0x80000000u) | 0x3f000000u);
+  return __builtin_truncf(__builtin_fmaf(x, rs, half));
+}
+
+// Quantize one gathered block (32 floats holding bf16 values) into packed codes.
+template <int FMT>
+__device__ __forceinline__ int quantize_block(const float (&f)[32], unsigned (&out)[8]) {
+  float amax = 0.0f;
+#pragma unroll
+  for (int p = 0; p < 32; p += 2) amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(f[p]), __builtin_fabsf(f[p + 1])));
+  const int byte = scale_byte<FMT>(amax);
+  const float rs = __uint_as_float((unsigned)(254 - byte) << 23);
+  float v[32];
+#pragma unroll
+  for (int p = 0; p < 32; ++p) v[p] = round_scaled(f[p], rs);
+
+  if constexpr (FMT == kFmtE2M1) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      unsigned w = 0;
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, v[8 * j + 0], v[8 * j + 1], 1.0f, 0);
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, v[8 * j + 2], v[8 * j + 3], 1.0f, 1);
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, v[8 * j + 4], v[8 * j + 5], 1.0f, 2);
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, v[8 * j + 6], v[8 * j + 7], 1.0f, 3);
+      out[j] = w;
+    }
+  } else if constexpr (FMT == kFmtE3M2) {
+    v32bf h;
+#pragma unroll
+    for (int p = 0; p < 32; ++p) h[p] = (__bf16)v[p];
+    // the ISA calls E3M2 "bf6" (its "fp6" is E2M3)
+    v6u w = __builtin_amdgcn_cvt_scalef32_pk32_bf6_bf16(h, 1.0f);
+#pragma unroll
+    for (int j = 0; j < 6; ++j) out[j] = w[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // the bf16 hop of the reference (src/reorder.cu:223) is a real rounding above 256
+      v2bf lo = {(__bf16)v[4 * j + 0], (__bf16)v[4 * j + 1]};
+      v2bf hi = {(__bf16)v[4 * j + 2], (__bf16)v[4 * j + 3]};
+      v2s z = {0, 0};
+      z = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(z, lo, 1.0f, false);
+      z = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(z, hi, 1.0f, true);
+      out[j] = __builtin_bit_cast(unsigned, z);
+    }
+  }
+  return byte;
+}
+
+template <int FMT>
+__device__ __forceinline__ void quantize_store(const float (&f)[32], uint8_t* __restrict__ q, uint8_t* __restrict__ sf) {
+  unsigned out[8];
+  const int byte = quantize_block<FMT>(f, out);
+  if constexpr (FMT == kFmtE2M1) {
+    *reinterpret_cast<v4u*>(q) = v4u{out[0], out[1], out[2], out[3]};
+  } else if constexpr (FMT == kFmtE3M2) {
+    v2u* p = reinterpret_cast<v2u*>(q);
+    p[0] = v2u{out[0], out[1]};
+    p[1] = v2u{out[2], out[3]};
+    p[2] = v2u{out[4], out[5]};
+  } else {
+    v4u* p = reinterpret_cast<v4u*>(q);
+    p[0] = v4u{out[0], out[1], out[2], out[3]};
+    p[1] = v4u{out[4], out[5], out[6], out[7]};
+  }
+  *sf = (uint8_t)byte;
+}
+
+// One workgroup handles R consecutive rows; blockDim.x >= K/32.
+template <int R, bool IS_W>
+__global__ void __launch_bounds__(1024)
+reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__ idx, int rows, int K, int KN, int KS,
+                     int KO, uint8_t* __restrict__ qn, uint8_t* __restrict__ qs, uint8_t* __restrict__ qo,
+                     uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const int tid = threadIdx.x;
+  const int nthr = blockDim.x;
+  const int row0 = blockIdx.x * R;
+
+  // ---- stage R rows: coalesced 16-byte loads, R x 8 transpose in registers,
+  //      16-byte LDS stores.  Channel c of row r lands at lds[(c*R + r)*2].
+  const int nchunks = K >> 3;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int c = tid + it * nthr;
+    if (c < nchunks) {
+      v4u a[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        a[r] = v4u{0, 0, 0, 0};
+        if (row0 + r < rows) a[r] = *reinterpret_cast<const v4u*>(x + (size_t)(row0 + r) * K + (size_t)c * 8);
+      }
+      v4u* dst = reinterpret_cast<v4u*>(lds + (size_t)c * 16 * R);
+      if constexpr (R == 1) {
+        dst[0] = a[0];
+      } else if constexpr (R == 2) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          v4u o;
+          o[0] = perm(a[1][2 * h], a[0][2 * h], 0x05040100u);
+          o[1] = perm(a[1][2 * h], a[0][2 * h], 0x07060302u);
+          o[2] = perm(a[1][2 * h + 1], a[0][2 * h + 1], 0x05040100u);
+          o[3] = perm(a[1][2 * h + 1], a[0][2 * h + 1], 0x07060302u);
+          dst[h] = o;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v4u o;
+          o[0] = perm(a[1][j], a[0][j], 0x05040100u);
+          o[1] = perm(a[3][j], a[2][j], 0x05040100u);
+          o[2] = perm(a[1][j], a[0][j], 0x07060302u);
+          o[3] = perm(a[3][j], a[2][j], 0x07060302u);
+          dst[j] = o;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- one lane per 32-element block
+  const int b = tid;
+  if (b >= (K >> 5)) return;
+  const int nbn = KN >> 5, nbs = KS >> 5;
+  const int seg = b < nbn ? 0 : (b < nbn + nbs ? 1 : 2);
+  const int j = seg == 0 ? b : (seg == 1 ? b - nbn : b - nbn - nbs);
+  const int kseg = seg == 0 ? KN : (seg == 1 ? KS : KO);
+  const int katoms = (kseg + 127) >> 7;
+
+  unsigned g[32][(R + 1) / 2];
+  {
+    const v4u* ip = reinterpret_cast<const v4u*>(idx + (size_t)b * 32);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const v4u iv = ip[q];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const unsigned ch = (e & 1) ? (iv[e >> 1] >> 16) : (iv[e >> 1] & 0xffffu);
+        const int p = q * 8 + e;
+        if constexpr (R == 4) {
+          const v2u d = *reinterpret_cast<const v2u*>(lds + ch * 8);
+          g[p][0] = d[0];
+          g[p][1] = d[1];
+        } else if constexpr (R == 2) {
+          g[p][0] = *reinterpret_cast<const unsigned*>(lds + ch * 4);
+        } else {
+          g[p][0] = *reinterpret_cast<const uint16_t*>(lds + ch * 2);
+        }
+      }
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int row = row0 + r;
+    if (row >= rows) break;
+    float f[32];
+#pragma unroll
+    for (int p = 0; p < 32; ++p) {
+      const unsigned d = g[p][r >> 1];
+      f[p] = __uint_as_float((r & 1) ? (d & 0xffff0000u) : (d << 16));
+    }
+    if (seg == 0) {
+      quantize_store<kFmtE2M1>(f, qn + (size_t)row * (KN >> 1) + j * 16, sfn + sf_offset(row, j, katoms));
+    } else if (seg == 1) {
+      if constexpr (IS_W)
+        quantize_store<kFmtE2M1>(f, qs + (size_t)row * (KS >> 1) + j * 16, sfs + sf_offset(row, j, katoms));
+      else
+        quantize_store<kFmtE3M2>(f, qs + (size_t)row * (KS / 4 * 3) + j * 24, sfs + sf_offset(row, j, katoms));
+    } else {
+      if constexpr (IS_W)
+        quantize_store<kFmtE2M1>(f, qo + (size_t)row * (KO >> 1) + j * 16, sfo + sf_offset(row, j, katoms));
+      else
+        quantize_store<kFmtE4M3>(f, qo + (size_t)row * KO + j * 32, sfo + sf_offset(row, j, katoms));
+    }
+  }
+}
+
+}  // namespace
+
+template <bool IS_W>
+hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int K, int KN, int KS, int KO, uint8_t* qn,
+                                uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo,
+                                hipStream_t stream) {
+  if (rows == 0 || K == 0) return hipSuccess;
+  const int threads = ((K >> 5) + 63) & ~63;
+  const uint16_t* xb = static_cast<const uint16_t*>(x);
+  // R rows interleaved in LDS; keep the tile within 64 KB so several workgroups share a CU
+  if (K <= 8192) {
+    hipLaunchKernelGGL((reorder_quant_kernel<4, IS_W>), dim3(ceil_div(rows, 4)), dim3(threads), (size_t)K * 8, stream, xb,
+                       idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+  } else if (K <= 16384) {
+    hipLaunchKernelGGL((reorder_quant_kernel<2, IS_W>), dim3(ceil_div(rows, 2)), dim3(threads), (size_t)K * 4, stream, xb,
+                       idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+  } else {
+    hipLaunchKernelGGL((reorder_quant_kernel<1, IS_W>), dim3(rows), dim3(threads), (size_t)K * 2, stream, xb, idx, rows, K,
+                       KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+  }
+  return hipGetLastError();
+}
+
+template hipError_t launch_reorder_quant<false>(const void*, const int16_t*, int, int, int, int, int, uint8_t*, uint8_t*,
+                                                uint8_t*, uint8_t*, uint8_t*, uint8_t*, hipStream_t);
+template hipError_t launch_reorder_quant<true>(const void*, const int16_t*, int, int, int, int, int, uint8_t*, uint8_t*,
+                                               uint8_t*, uint8_t*, uint8_t*, uint8_t*, hipStream_t);
+
+}  // namespace mg

@@ -164,7 +164,7 @@ def pack_fp4(codes: np.ndarray) -> np.ndarray:
     """[..., n] 4-bit codes -> [..., n/2] bytes, even element in the low nibble
     (src/reorder.cu:30-33,243-246)."""
     c = np.asarray(codes, dtype=np.uint8)
-    return (c[..., 0::2] & 0xF) | ((c[..., 1::2] & 0xF) << 4)
+    return np.ascontiguousarray((c[..., 0::2] & 0xF) | ((c[..., 1::2] & 0xF) << 4))
 
 
 def unpack_fp4(b: np.ndarray) -> np.ndarray:
@@ -251,7 +251,7 @@ def reorder_quantize_x(x: np.ndarray, idx: np.ndarray, kn: int, ks: int, ko: int
     logical (unpacked) codes / scale bytes."""
     x = np.asarray(x, dtype=np.float32)
     m = x.shape[0]
-    xr = x[:, np.asarray(idx, dtype=np.int64)]
+    xr = np.ascontiguousarray(x[:, np.asarray(idx, dtype=np.int64)])
     out = {}
     for name, fmt, (lo, hi), pack in zip(
         ("n", "s", "o"), ("e2m1", "e3m2", "e4m3"), _segments(kn, ks, ko),
@@ -272,7 +272,7 @@ def reorder_quantize_w(w: np.ndarray, idx: np.ndarray, kn: int, ks: int, ko: int
     segment quantized to E2M1."""
     w = np.asarray(w, dtype=np.float32)
     n = w.shape[0]
-    wr = w[:, np.asarray(idx, dtype=np.int64)]
+    wr = np.ascontiguousarray(w[:, np.asarray(idx, dtype=np.int64)])
     out = {}
     for name, (lo, hi) in zip(("n", "s", "o"), _segments(kn, ks, ko)):
         kseg = hi - lo

@@ -1,0 +1,102 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every
+symbol the header declares, and its host logic (sizes, offsets, validation that
+happens before any launch) agrees with the oracle."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import mx_oracle as mo
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mixedgemm_abi.h")
+
+
+@pytest.fixture(scope="module")
+def abi():
+    from mixedgemm_amd import abi as a
+    if not os.path.exists(a.LIB_PATH):
+        from mixedgemm_amd import build
+        build.build_hip_library()
+    return a
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(abi):
+    lib = ctypes.CDLL(abi.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 9
+    for name in names:
+        assert hasattr(lib, name), name
+    assert set(names) == set(abi.SYMBOLS)
+
+
+@pytest.mark.parametrize("rows,kseg", [(114, 2560), (4096, 1408), (8, 128), (2048, 4928), (2048, 448), (1, 32), (0, 128)])
+def test_sf_bytes_and_offsets_match_oracle(abi, rows, kseg):
+    assert abi.sf_bytes(rows, kseg, abi.MG_OPERAND_A) == mo.sf_bytes(rows, kseg, "a")
+    assert abi.sf_bytes(rows, kseg, abi.MG_OPERAND_B) == mo.sf_bytes(rows, kseg, "b")
+    rng = np.random.default_rng(rows + kseg)
+    for _ in range(50):
+        r, kb = int(rng.integers(0, max(rows, 1))), int(rng.integers(0, kseg // 32))
+        assert abi.sf_offset(r, kb, kseg) == int(mo.sf_offset(r, kb, kseg))
+
+
+def test_validation_rejects_bad_shapes_before_any_launch(abi):
+    lib = abi.lib()
+    null = ctypes.c_void_p(0)
+    args = [null] * 6
+    # a segment that is not a multiple of 32
+    assert lib.mg_reorder_quantize_x(null, null, 4, 4096, 2560, 1400, 136, *args, null) == 10001
+    # K != KN + KS + KO
+    assert lib.mg_reorder_quantize_w(null, null, 4, 4000, 2560, 1408, 128, *args, null) == 10001
+    # K beyond the int16 index range
+    assert lib.mg_reorder_quantize_x(null, null, 4, 32768, 32768, 0, 0, *args, null) == 10004
+    # null pointers with a non-empty problem
+    assert lib.mg_reorder_quantize_x(null, null, 4, 4096, 2560, 1408, 128, *args, null) == 10002
+    assert lib.mg_mixed_gemm(*([null] * 12), 4, 8, 128, 0, 0, null, null) == 10002
+    # empty problems succeed without touching the device
+    assert lib.mg_reorder_quantize_x(null, null, 0, 4096, 2560, 1408, 128, *args, null) == 0
+    assert lib.mg_mixed_gemm(*([null] * 12), 0, 8, 128, 0, 0, null, null) == 0
+    assert "multiples of 32" in abi.status_string(10001)
+
+
+def test_fused_workspace_size(abi):
+    m, kn, ks, ko = 4096, 2560, 1408, 128
+    need = abi.fused_workspace_bytes(m, kn, ks, ko)
+    parts = [m * kn // 2, m * ks * 3 // 4, m * ko] + [mo.sf_bytes(m, k, "a") for k in (kn, ks, ko)]
+    assert need == sum((p + 255) // 256 * 256 for p in parts)
+
+
+def test_extension_module_surface():
+    """The torch extension keeps the reference's operator names and keywords."""
+    import sys
+    ext = os.path.join(ROOT, "build", "mixedgemm.so")
+    if not os.path.exists(ext):
+        from mixedgemm_amd import build
+        build.build_all()
+    sys.path.insert(0, os.path.join(ROOT, "build"))
+    import torch  # noqa: F401  (the extension links against libtorch)
+    import mixedgemm
+    assert mixedgemm.test_function() == "Hello from test_function!"
+    for name in ("matmul", "reorder_quantize_x", "reorder_quantize_w"):
+        assert callable(getattr(mixedgemm, name))
+    doc = mixedgemm.reorder_quantize_x.__doc__
+    for kw in ("X", "reorder_index", "KN", "KS", "KO", "seqlen", "outfeatures"):
+        assert kw in doc
+    doc = mixedgemm.matmul.__doc__
+    for kw in ("AN", "BN", "AS", "BS", "AO", "BO", "SFAN", "SFBN", "SFAS", "SFBS", "SFAO", "SFBO"):
+        assert kw in doc
+    # invalid K: same exception type and message as the reference boundary
+    x = torch.zeros(2, 100, dtype=torch.bfloat16)
+    idx = torch.arange(100, dtype=torch.int16)
+    with pytest.raises(RuntimeError, match="Value error in run_reorder_bf16_mixed"):
+        mixedgemm.reorder_quantize_x(x, idx, 50, 30, 20, 2, 2)
+    with pytest.raises(RuntimeError, match="Value error in run_reorder_bf16_fp4"):
+        mixedgemm.reorder_quantize_w(x, idx, 50, 30, 20, 2, 2)

@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the hot path over configuration c3 of BASELINE.json:
+activation reorder-quantize (bf16 [4096, 4096] -> packed MXFP4/6/8 + E8M0
+scales) followed by the mixed GEMM against MXFP4 weights [14336, 4096] into bf16
+[4096, 14336], with every input already resident in HBM and the weights quantized
+once outside the timed region (as bench_reorder_gemm.cu:163-167 of the reference
+does).  Prints ONE JSON line.  `roofline` describes the dominant kernel (the mixed
+GEMM, MFMA-bound); `extra` carries the memory-bound configurations c1 (reorder-
+quantize alone) and c2 (decode GEMM) with their own rooflines; `cpu_baseline` is
+the oracle's fake-quant + fp32 matmul timed on the host cores over a bounded
+sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+# dense MFMA peaks, TFLOP/s: an E4M3 operand halves the f8f6f4 rate
+P46, P8 = 10100.0, 5000.0
+
+
+def blended_peak(kn, ks, ko):
+    return (kn + ks + ko) / ((kn + ks) / P46 + ko / P8)
+
+
+def quant_bytes(m, k, kn, ks, ko):
+    """Algorithmic bytes of one activation reorder-quantize launch."""
+    return m * (2 * k + kn // 2 + 3 * ks // 4 + ko + k // 32) + 2 * k
+
+
+def gemm_bytes(m, n, kn, ks, ko):
+    k = kn + ks + ko
+    return n * k // 2 + n * k // 32 + m * (kn // 2 + 3 * ks // 4 + ko) + m * k // 32 + m * n * 2
+
+
+def event_ms(pairs):
+    return sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from mixedgemm_amd import abi
+    from tests import helpers as H
+
+    abi.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---------------------------------------------------------------- c3
+    m, n, k, kn, ks, ko = H.CONFIGS["c3"]
+    x = H.make_activations(m, k, 1234 + 3)
+    w = H.make_weights(n, k, 2234 + 3)
+    idx = H.absmax_sort_index(x)
+    xd, wd, idd = x.to(dev), w.to(dev), idx.to(dev)
+    bq = abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+    aq = abi.alloc_quant_outputs(m, kn, ks, ko, abi.MG_OPERAND_A, dev)
+    d = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+
+    def step(pair=None):
+        abi.reorder_quantize_x(xd, idd, kn, ks, ko, out=aq)
+        if pair:
+            pair[0].record()
+        abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], out=d)
+        if pair:
+            pair[1].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(ev[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    flops = 2.0 * m * n * k
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    gemm_ms = event_ms(ev)
+    peak = blended_peak(kn, ks, ko)
+    gemm_tflops = flops / (gemm_ms * 1e-3) / 1e12
+    roofline = {
+        "kernel": "mixed GEMM (c3)", "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": round(peak, 1),
+        "unit": "TFLOP/s", "frac": round(gemm_tflops / peak, 4), "traffic": None,
+        "avg_kernel_ms": round(gemm_ms, 4), "algorithmic_flops": flops,
+    }
+
+    extra = {}
+    if not args.no_extra:
+        # ------------------------------------------------------------ c1: reorder-quantize alone, HBM-bound
+        m1, _, k1, kn1, ks1, ko1 = H.CONFIGS["c1"]
+        nsets = 8                                    # 8 x 44 MB > 256 MB Infinity Cache
+        idx1 = H.random_index(k1, 4321).to(dev)
+        base = H.make_activations(m1, k1, 1234 + 1).to(dev)
+        xs = [base.clone() for _ in range(nsets)]
+        outs = [abi.alloc_quant_outputs(m1, kn1, ks1, ko1, abi.MG_OPERAND_A, dev) for _ in range(nsets)]
+        iters = max(args.steps, 40)
+        for i in range(args.warmup + nsets):
+            abi.reorder_quantize_x(xs[i % nsets], idx1, kn1, ks1, ko1, out=outs[i % nsets])
+        torch.cuda.synchronize()
+        ev1 = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        for i in range(iters):
+            ev1[i][0].record()
+            abi.reorder_quantize_x(xs[i % nsets], idx1, kn1, ks1, ko1, out=outs[i % nsets])
+            ev1[i][1].record()
+        torch.cuda.synchronize()
+        q_ms = event_ms(ev1)
+        qb = quant_bytes(m1, k1, kn1, ks1, ko1)
+        q_gbs = qb / (q_ms * 1e-3) / 1e9
+        extra["reorder_quant_c1"] = {
+            "workload": "c1 reorder-quantize M=4096 K=4096 (2560/1408/128), random-permutation index, 8 rotating buffer sets",
+            "value": round(q_gbs, 1), "unit": "GB/s", "avg_kernel_ms": round(q_ms, 5),
+            "roofline": {"bound": "hbm", "achieved": round(q_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": qb},
+        }
+        del xs, outs, base
+
+        # ------------------------------------------------------------ c2: decode GEMM, HBM-bound
+        m2, n2, k2, kn2, ks2, ko2 = H.CONFIGS["c2"]
+        x2 = H.make_activations(m2, k2, 1234 + 2)
+        idx2 = H.absmax_sort_index(x2).to(dev)
+        aq2 = abi.reorder_quantize_x(x2.to(dev), idx2, kn2, ks2, ko2)
+        nsets2 = 10                                  # 10 x 31 MB of weights > 256 MB
+        wq = [abi.reorder_quantize_w(H.make_weights(n2, k2, 3000 + i).to(dev), idx2, kn2, ks2, ko2) for i in range(nsets2)]
+        d2 = torch.empty((m2, n2), dtype=torch.bfloat16, device=dev)
+        for i in range(args.warmup + nsets2):
+            b = wq[i % nsets2]
+            abi.matmul(aq2[0], b[0], aq2[1], b[1], aq2[2], b[2], aq2[3], b[3], aq2[4], b[4], aq2[5], b[5], out=d2)
+        torch.cuda.synchronize()
+        ev2 = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        for i in range(iters):
+            b = wq[i % nsets2]
+            ev2[i][0].record()
+            abi.matmul(aq2[0], b[0], aq2[1], b[1], aq2[2], b[2], aq2[3], b[3], aq2[4], b[4], aq2[5], b[5], out=d2)
+            ev2[i][1].record()
+        torch.cuda.synchronize()
+        g_ms = event_ms(ev2)
+        gb = gemm_bytes(m2, n2, kn2, ks2, ko2)
+        g_gbs = gb / (g_ms * 1e-3) / 1e9
+        extra["decode_gemm_c2"] = {
+            "workload": "c2 mixed GEMM M=8 K=4096 (2560/1408/128) N=14336, 10 rotating weight sets",
+            "value": round(g_gbs, 1), "unit": "GB/s", "avg_kernel_ms": round(g_ms, 5),
+            "tflops": round(2.0 * m2 * n2 * k2 / (g_ms * 1e-3) / 1e12, 3),
+            "roofline": {"bound": "hbm", "achieved": round(g_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(g_gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": gb},
+        }
+        del wq
+
+    # ---------------------------------------------------------------- CPU baseline (oracle, host cores)
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import mx_oracle as mo
+        from oracle import scalar as sc
+        torch_threads = torch.get_num_threads()
+        rows = 256
+        wq_host = sc.quantize_w(H.bf16_bits(w), idx.numpy(), kn, ks, ko)          # offline, as on the GPU
+        wdeq = torch.from_numpy(np.concatenate([
+            mo.dequantize(mo.unpack_fp4(wq_host[q]), mo.sf_gather(wq_host[s], n, kk), "e2m1")
+            for q, s, kk in (("qn", "sfn", kn), ("qs", "sfs", ks), ("qo", "sfo", ko))], axis=1))
+        xs_bits = H.bf16_bits(x[:rows])
+
+        def cpu_step():
+            q = sc.quantize_x(xs_bits, idx.numpy(), kn, ks, ko)
+            xdeq = np.concatenate([
+                mo.dequantize(mo.unpack_fp4(q["qn"]), mo.sf_gather(q["sfn"], rows, kn), "e2m1"),
+                mo.dequantize(mo.unpack_fp6(q["qs"]), mo.sf_gather(q["sfs"], rows, ks), "e3m2"),
+                mo.dequantize(q["qo"], mo.sf_gather(q["sfo"], rows, ko), "e4m3")], axis=1)
+            return (torch.from_numpy(xdeq) @ wdeq.T).to(torch.bfloat16)
+
+        cpu_step()
+        reps = 3
+        c0 = time.perf_counter()
+        for _ in range(reps):
+            cpu_step()
+        c_s = (time.perf_counter() - c0) / reps
+        cpu = {
+            "value": round(2.0 * rows * n * k / c_s / 1e12, 4), "unit": "TFLOP/s",
+            "cores": torch_threads, "kind": "port",
+            "sample": f"first {rows} of {m} token rows of c3 (full N={n}, K={k}): C-oracle reorder-quantize + NumPy "
+                      f"dequantize + torch fp32 matmul, weights quantized offline; 1 warm-up + {reps} repeats; "
+                      f"os.cpu_count()={os.cpu_count()}",
+        }
+        if "reorder_quant_c1" in extra:
+            m1, _, k1, kn1, ks1, ko1 = H.CONFIGS["c1"]
+            r1 = 1024
+            x1b = H.bf16_bits(H.make_activations(m1, k1, 1234 + 1)[:r1])
+            i1 = H.random_index(k1, 4321).numpy()
+            sc.quantize_x(x1b, i1, kn1, ks1, ko1)
+            c0 = time.perf_counter()
+            for _ in range(reps):
+                sc.quantize_x(x1b, i1, kn1, ks1, ko1)
+            c1_s = (time.perf_counter() - c0) / reps
+            extra["reorder_quant_c1"]["cpu_baseline"] = {
+                "value": round(quant_bytes(r1, k1, kn1, ks1, ko1) / c1_s / 1e9, 3), "unit": "GB/s",
+                "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count())), "kind": "port",
+                "sample": f"first {r1} of {m1} rows of c1, scalar C oracle with OpenMP over rows",
+            }
+
+    out = {
+        "metric": "mixed_mx_gemm_tflops", "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "mxfp4/mxfp6/mxfp8 x mxfp4 -> f32 accumulate -> bf16", "data": "synthetic",
+        "config": {"workload": "c3 prefill: reorder-quantize bf16 X[4096,4096] + mixed GEMM vs MXFP4 W[14336,4096] "
+                               "(K split 2560 fp4 / 1408 fp6 / 128 fp8), bf16 out",
+                   "M": m, "N": n, "K": k, "KN": kn, "KS": ks, "KO": ko},
+        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

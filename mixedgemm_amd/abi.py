@@ -91,34 +91,42 @@ def _require(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
         raise MixedGemmError(f"{name}: expected a contiguous tensor")
 
 
-def _reorder_quantize(fn_name, operand, t, idx, kn, ks, ko):
+def alloc_quant_outputs(rows, kn, ks, ko, operand, device):
+    """The six output tensors of a reorder-quantize call (codes x3, scales x3)."""
+    w = operand == MG_OPERAND_B
+    u8 = dict(dtype=torch.uint8, device=device)
+    return (torch.empty((rows, kn // 2), **u8),
+            torch.empty((rows, ks // 2 if w else ks // 4 * 3), **u8),
+            torch.empty((rows, ko // 2 if w else ko), **u8),
+            torch.empty(sf_bytes(rows, kn, operand), **u8),
+            torch.empty(sf_bytes(rows, ks, operand), **u8),
+            torch.empty(sf_bytes(rows, ko, operand), **u8))
+
+
+def _reorder_quantize(fn_name, operand, t, idx, kn, ks, ko, out=None):
     _require(t, torch.bfloat16, "input")
     _require(idx, torch.int16, "reorder_index")
     rows, k = t.shape
     if idx.numel() != k:
         raise MixedGemmError(f"reorder_index has {idx.numel()} entries, input has {k} channels")
-    w = operand == MG_OPERAND_B
-    u8 = dict(dtype=torch.uint8, device=t.device)
-    qn = torch.empty((rows, kn // 2), **u8)
-    qs = torch.empty((rows, ks // 2 if w else ks // 4 * 3), **u8)
-    qo = torch.empty((rows, ko // 2 if w else ko), **u8)
-    sfn = torch.empty(sf_bytes(rows, kn, operand), **u8)
-    sfs = torch.empty(sf_bytes(rows, ks, operand), **u8)
-    sfo = torch.empty(sf_bytes(rows, ko, operand), **u8)
+    if out is None:
+        out = alloc_quant_outputs(rows, kn, ks, ko, operand, t.device)
+    qn, qs, qo, sfn, sfs, sfo = out
     status = getattr(lib(), fn_name)(_ptr(t), _ptr(idx), rows, k, kn, ks, ko,
                                      _ptr(qn), _ptr(qs), _ptr(qo), _ptr(sfn), _ptr(sfs), _ptr(sfo), _stream(t))
     check(status, fn_name)
     return qn, qs, qo, sfn, sfs, sfo
 
 
-def reorder_quantize_x(x, reorder_index, kn, ks, ko):
-    """(XN, XS, XO, SFXN, SFXS, SFXO); asynchronous on torch's current stream."""
-    return _reorder_quantize("mg_reorder_quantize_x", MG_OPERAND_A, x, reorder_index, kn, ks, ko)
+def reorder_quantize_x(x, reorder_index, kn, ks, ko, out=None):
+    """(XN, XS, XO, SFXN, SFXS, SFXO); asynchronous on torch's current stream.
+    `out` may carry six preallocated tensors (see alloc_quant_outputs)."""
+    return _reorder_quantize("mg_reorder_quantize_x", MG_OPERAND_A, x, reorder_index, kn, ks, ko, out)
 
 
-def reorder_quantize_w(w, reorder_index, kn, ks, ko):
+def reorder_quantize_w(w, reorder_index, kn, ks, ko, out=None):
     """(WN, WS, WO, SFWN, SFWS, SFWO); asynchronous on torch's current stream."""
-    return _reorder_quantize("mg_reorder_quantize_w", MG_OPERAND_B, w, reorder_index, kn, ks, ko)
+    return _reorder_quantize("mg_reorder_quantize_w", MG_OPERAND_B, w, reorder_index, kn, ks, ko, out)
 
 
 def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None):

@@ -146,15 +146,29 @@ mixed_gemm_direct_kernel(const uint8_t* __restrict__ an, const uint8_t* __restri
 // Workgroup = 4 waves = 256 features x 128 tokens; wave = 128 x 64 (4 x 2 MFMA
 // tiles, 128 accumulator registers), two workgroups per CU so one covers the
 // other's barrier and memory stalls.  One K stage = 128 elements = one dword of
-// scales per row = two MFMA K steps.  Operand tiles go global -> registers ->
-// LDS (double buffered) in a fragment-major order: the 16/24 bytes a lane feeds
-// to one MFMA lie at (lane * 16 or 24) inside a 1 KB / 1.5 KB fragment, so every
-// fragment read is one linear, conflict-free pass over LDS.
+// scales per row = two MFMA K steps; LDS is double buffered.
+//
+// Every operand byte goes global -> LDS directly (global_load_lds_dwordx4: no
+// staging registers, no LDS store instructions).  One such instruction moves
+// 64 x 16 B to 1 KB of consecutive LDS; each lane quad reads 64 (or 96)
+// contiguous bytes of one row.  Which rows an instruction gathers, and where its
+// block sits, is chosen so that the 16 lanes that fetch rows 32t..32t+15 of a
+// fragment land in 16 different banks groups:
+//   weights (64 B rows):  instruction j moves rows j, j+16, ..., j+240; block j
+//                         at j*1040, so those lanes are 65 slots of 16 B apart;
+//   E2M1 / E4M3 tokens:   instruction j moves rows j + 8t, t = 0..15, row t at
+//                         quad 4*(t/4) + tau(t%4), tau = (0,2,1,3); block j at
+//                         j*1040 (E4M3: one set of blocks per 64-wide K half);
+//   E3M2 tokens (96 B):   three instructions move rows j + 4t, t = 0..31, as one
+//                         row-major block of 3072 B at j*3088.
+// The scale atoms (512 B per 128 rows per stage) are copied the same way.
 // ---------------------------------------------------------------------------
 constexpr int kTileN = 256, kTileM = 128, kStageK = 128;
-constexpr int kWBytes = kTileN * 64;           // weights, E2M1: 64 B per row per stage
-constexpr int kXBytesMax = kTileM * 128;       // activations, E4M3 worst case
-constexpr int kStageBytes = kWBytes + kXBytesMax;
+constexpr int kBlock = 1040;                   // 16 rows x 64 B + 16 B of padding
+constexpr int kWBytes = 16 * kBlock;           // weights, E2M1: 64 B per row per stage
+constexpr int kXBytes = 16 * kBlock;           // activations, E4M3 worst case (E3M2: 4 * 3088)
+constexpr int kSBytes = 1024 + 512;            // two weight scale atoms + one activation scale atom
+constexpr int kStageBytes = kWBytes + kXBytes + kSBytes;
 
 struct Seg {
   const uint8_t* a;    // activation codes of the segment
@@ -169,174 +183,178 @@ template <> struct RowBytes<kFmtE2M1> { static constexpr int v = 64; };
 template <> struct RowBytes<kFmtE3M2> { static constexpr int v = 96; };
 template <> struct RowBytes<kFmtE4M3> { static constexpr int v = 128; };
 
-struct Staging {
-  v4i w[4];
-  v4i x[4];
-  v4i sw, sx;   // scale dwords of the wave's row tiles for the staged K stage
-};
+typedef int v6i __attribute__((ext_vector_type(6)));
+template <int FMT> struct XFrag;      // registers of one activation fragment
+template <> struct XFrag<kFmtE2M1> { typedef v4i type; };
+template <> struct XFrag<kFmtE3M2> { typedef v6i type; };
+template <> struct XFrag<kFmtE4M3> { typedef v8i type; };
 
-// Per-thread byte offsets of the 16-byte chunks a thread copies each stage,
-// relative to the (uniform) start of the tile's rows in the current stage.
-template <int FMT>
-struct LoadOffsets {
-  unsigned w;      // weight chunk k lives at w + k * 64 rows
-  unsigned x[3];   // E2M1: x[0] + k * 64 rows; E3M2: x[k]; E4M3: x[0] + k * 32 rows
-  __device__ __forceinline__ LoadOffsets(int tid, unsigned ldb, unsigned lda) {
-    w = (unsigned)(tid >> 2) * ldb + (tid & 3) * 16;
-    if constexpr (FMT == kFmtE2M1) {
-      x[0] = (unsigned)(tid >> 2) * lda + (tid & 3) * 16;
-    } else if constexpr (FMT == kFmtE3M2) {
-#pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        const int id = tid + 256 * k;
-        x[k] = (unsigned)(id / 6) * lda + (id % 6) * 16;
-      }
-    } else {
-      x[0] = (unsigned)(tid >> 3) * lda + (tid & 7) * 16;
-    }
-  }
-};
+__device__ __forceinline__ v8i widen(v4i v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1); }
+__device__ __forceinline__ v8i widen(v6i v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3, 4, 5, -1, -1); }
+__device__ __forceinline__ v8i widen(v8i v) { return v; }
 
-// global -> registers for K stage `q` of a segment
-template <int FMT>
-__device__ __forceinline__ void stage_load(Staging& st, const Seg& sg, int q, int n0, int m0, int tid, int lane, int wn,
-                                           int wm) {
-  constexpr int RB = RowBytes<FMT>::v;
-  const int nst = sg.stages;
-  const unsigned ldb = (unsigned)nst * 64, lda = (unsigned)nst * RB;
-  const LoadOffsets<FMT> off(tid, ldb, lda);
-  const uint8_t* wbase = sg.b + (size_t)n0 * ldb + (size_t)q * 64;
-#pragma unroll
-  for (int k = 0; k < 4; ++k) st.w[k] = *reinterpret_cast<const v4i*>(wbase + (size_t)k * 64 * ldb + off.w);
-  const uint8_t* xbase = sg.a + (size_t)m0 * lda + (size_t)q * RB;
-  if constexpr (FMT == kFmtE2M1) {
-#pragma unroll
-    for (int k = 0; k < 2; ++k) st.x[k] = *reinterpret_cast<const v4i*>(xbase + (size_t)k * 64 * lda + off.x[0]);
-  } else if constexpr (FMT == kFmtE3M2) {
-#pragma unroll
-    for (int k = 0; k < 3; ++k) st.x[k] = *reinterpret_cast<const v4i*>(xbase + off.x[k]);
-  } else {
-#pragma unroll
-    for (int k = 0; k < 4; ++k) st.x[k] = *reinterpret_cast<const v4i*>(xbase + (size_t)k * 32 * lda + off.x[0]);
-  }
-  // scales: the wave's 128 feature rows are one 512-byte atom, its 64 token rows half of one;
-  // lane i reads the 16 bytes that hold the dwords of rows i, 32+i, 64+i, 96+i
-  const unsigned i16 = (lane & 31) * 16;
-  st.sw = *reinterpret_cast<const v4i*>(sg.sfb + ((size_t)((n0 >> 7) + wn) * nst + q) * 512 + i16);
-  st.sx = *reinterpret_cast<const v4i*>(sg.sfa + ((size_t)(m0 >> 7) * nst + q) * 512 + i16);
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+__device__ __forceinline__ void copy16(const uint8_t* base, unsigned off, uint8_t* lds_dst) {
+  __builtin_amdgcn_global_load_lds(base + off, (lds_ptr)lds_dst, 16, 0, 0);
 }
 
-// registers -> LDS, fragment-major
+__device__ __forceinline__ int tau(int e) { return ((e & 1) << 1) | (e >> 1); }   // (0,2,1,3)
+
+// Per-lane byte offsets into the operand rows, fixed for a segment.
 template <int FMT>
-__device__ __forceinline__ void stage_store(const Staging& st, uint8_t* __restrict__ buf, int tid) {
+struct CopyOffsets {
+  unsigned w, x[3], s;
+  __device__ __forceinline__ CopyOffsets(const Seg& sg, int lane) {
+    const unsigned ldb = (unsigned)sg.stages * 64, lda = (unsigned)sg.stages * RowBytes<FMT>::v;
+    const int p = lane >> 2, c = lane & 3;
+    w = (unsigned)(16 * p) * ldb + c * 16;
+    if constexpr (FMT == kFmtE3M2) {
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        const int ci = 64 * k + lane;
+        x[k] = (unsigned)(4 * (ci / 6)) * lda + (ci % 6) * 16;
+      }
+    } else {
+      const int t = 4 * (p >> 2) + tau(p & 3);
+      x[0] = (unsigned)(8 * t) * lda + c * 16;
+    }
+    s = (unsigned)(lane >> 5) * sg.stages * 512 + (lane & 31) * 16;
+  }
+};
+
+// Issue the copies of K stage q of a segment into LDS buffer `buf`.  `wave` is uniform.
+template <int FMT>
+__device__ __forceinline__ void stage_copy(const Seg& sg, const CopyOffsets<FMT>& off, int q, int n0, int m0,
+                                           uint8_t* buf, int wave, int lane) {
+  constexpr int RB = RowBytes<FMT>::v;
+  const unsigned ldb = (unsigned)sg.stages * 64, lda = (unsigned)sg.stages * RB;
+  const uint8_t* wbase = sg.b + (size_t)n0 * ldb + (size_t)q * 64;
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    const int id = tid + 256 * k, row = id >> 2, c = id & 3;
-    // [row tile][h][g][i][16 B] with c = 2h + g
-    *reinterpret_cast<v4i*>(buf + (row >> 5) * 2048 + c * 512 + (row & 31) * 16) = st.w[k];
+    const int j = wave * 4 + k;
+    copy16(wbase + (size_t)j * ldb, off.w, buf + j * kBlock);
   }
+  const uint8_t* xbase = sg.a + (size_t)m0 * lda + (size_t)q * RB;
   uint8_t* xb = buf + kWBytes;
   if constexpr (FMT == kFmtE2M1) {
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-      const int id = tid + 256 * k, row = id >> 2, c = id & 3;
-      *reinterpret_cast<v4i*>(xb + (row >> 5) * 2048 + c * 512 + (row & 31) * 16) = st.x[k];
+      const int j = wave * 2 + k;
+      copy16(xbase + (size_t)j * lda, off.x[0], xb + j * kBlock);
     }
   } else if constexpr (FMT == kFmtE3M2) {
 #pragma unroll
-    for (int k = 0; k < 3; ++k) {
-      const int id = tid + 256 * k, row = id / 6, c = id % 6;
-      // 16-byte chunk c = 8-byte units 2c, 2c+1 of the row's 12; unit u belongs to fragment u/3
-      uint8_t* rb = xb + (row >> 5) * 3072 + (row & 31) * 24;
-      const int u0 = 2 * c, u1 = 2 * c + 1;
-      *reinterpret_cast<v2i*>(rb + (u0 / 3) * 768 + (u0 % 3) * 8) = v2i{st.x[k][0], st.x[k][1]};
-      *reinterpret_cast<v2i*>(rb + (u1 / 3) * 768 + (u1 % 3) * 8) = v2i{st.x[k][2], st.x[k][3]};
-    }
+    for (int k = 0; k < 3; ++k) copy16(xbase + (size_t)wave * lda, off.x[k], xb + wave * 3088 + k * 1024);
   } else {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      const int id = tid + 256 * k, row = id >> 3, c = id & 7;
-      // chunk c: K step h = c/4, piece (c%4)/2, lane group g = c%2 -> [row tile][h][piece][g][i][16 B]
-      *reinterpret_cast<v4i*>(xb + (row >> 5) * 4096 + (c >> 1) * 1024 + (c & 1) * 512 + (row & 31) * 16) = st.x[k];
+      const int id = wave * 4 + k, hh = id >> 3, j = id & 7;   // K half, row residue
+      copy16(xbase + (size_t)j * lda + hh * 64, off.x[0], xb + id * kBlock);
+    }
+  }
+  uint8_t* sb = buf + kWBytes + kXBytes;
+  if (wave == 0) {
+    copy16(sg.sfb + ((size_t)(n0 >> 7) * sg.stages + q) * 512, off.s, sb);
+  } else if (wave == 1) {
+    if (lane < 32) copy16(sg.sfa + ((size_t)(m0 >> 7) * sg.stages + q) * 512, off.s, sb + 1024);
+  }
+}
+
+// all fragments and scales of one stage: LDS -> registers
+template <int FMT>
+__device__ __forceinline__ void frags_read(v4i (&wf)[2][4], typename XFrag<FMT>::type (&xf)[2][2], v4i& sw, v4i& sx,
+                                           const uint8_t* __restrict__ buf, int lane, int wn, int wm) {
+  const int i = lane & 31, g = lane >> 5;
+  // row 32*rt + i of the weight tile: block i%16, quad 2*rt + i/16
+  const uint8_t* wl = buf + (i & 15) * kBlock + (i >> 4) * 64 + g * 16 + wn * 4 * 128;
+  const uint8_t* xb = buf + kWBytes;
+  const uint8_t* sb = buf + kWBytes + kXBytes;
+  sw = *reinterpret_cast<const v4i*>(sb + wn * 512 + i * 16);
+  sx = *reinterpret_cast<const v4i*>(sb + 1024 + i * 16);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) wf[h][t] = *reinterpret_cast<const v4i*>(wl + t * 128 + h * 32);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int rt = wm * 2 + t;
+      if constexpr (FMT == kFmtE2M1) {
+        // row 32*rt + i: block i%8, quad 4*rt + tau(i/8)
+        xf[h][t] = *reinterpret_cast<const v4i*>(xb + (i & 7) * kBlock + (4 * rt + tau(i >> 3)) * 64 + (2 * h + g) * 16);
+      } else if constexpr (FMT == kFmtE3M2) {
+        // row 32*rt + i: block i%4, row slot 8*rt + i/4, fragment 2h+g of 24 bytes
+        const v2i* p = reinterpret_cast<const v2i*>(xb + (i & 3) * 3088 + (8 * rt + (i >> 2)) * 96 + (2 * h + g) * 24);
+        const v2i a = p[0], b = p[1], c = p[2];
+        xf[h][t] = v6i{a[0], a[1], b[0], b[1], c[0], c[1]};
+      } else {
+        const uint8_t* p = xb + (h * 8 + (i & 7)) * kBlock + (4 * rt + tau(i >> 3)) * 64 + g * 16;
+        const v4i a = *reinterpret_cast<const v4i*>(p);        // K [16g, 16g+16) of the half
+        const v4i b = *reinterpret_cast<const v4i*>(p + 32);   // K [32+16g, 32+16g+16)
+        xf[h][t] = v8i{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+      }
     }
   }
 }
 
 template <int FMT>
-__device__ __forceinline__ void stage_compute(v16f (&acc)[4][2], const uint8_t* __restrict__ buf, v4i sw, v4i sx, int lane,
-                                              int wn, int wm) {
+__device__ __forceinline__ void stage_compute(v16f (&acc)[4][2], const v4i (&wf)[2][4],
+                                              const typename XFrag<FMT>::type (&xf)[2][2], v4i sw, v4i sx, int lane,
+                                              int wm) {
   const int g8 = (lane >> 5) * 8;
   int scw[4], scx[2];
 #pragma unroll
   for (int t = 0; t < 4; ++t) scw[t] = (int)((unsigned)sw[t] >> g8);
 #pragma unroll
-  for (int t = 0; t < 2; ++t) scx[t] = (int)((unsigned)sx[2 * wm + t] >> g8);
-  const uint8_t* wb = buf + wn * 4 * 2048 + lane * 16;
-  const uint8_t* xb = buf + kWBytes;
+  for (int t = 0; t < 2; ++t) scx[t] = (int)((unsigned)(wm ? sx[2 + t] : sx[t]) >> g8);
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    v8i wf[4], xf[2];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const v4i v = *reinterpret_cast<const v4i*>(wb + t * 2048 + h * 1024);
-      wf[t] = __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1);
-    }
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int rt = wm * 2 + t;
-      if constexpr (FMT == kFmtE2M1) {
-        const v4i v = *reinterpret_cast<const v4i*>(xb + rt * 2048 + h * 1024 + lane * 16);
-        xf[t] = __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1);
-      } else if constexpr (FMT == kFmtE3M2) {
-        const v2i* p = reinterpret_cast<const v2i*>(xb + rt * 3072 + h * 1536 + lane * 24);
-        const v2i a = p[0], b = p[1], c = p[2];
-        const v4i ab = __builtin_shufflevector(a, b, 0, 1, 2, 3);
-        const v4i cc = __builtin_shufflevector(c, c, 0, 1, -1, -1);
-        xf[t] = __builtin_shufflevector(ab, cc, 0, 1, 2, 3, 4, 5, -1, -1);
-      } else {
-        const v4i a = *reinterpret_cast<const v4i*>(xb + rt * 4096 + h * 2048 + lane * 16);
-        const v4i b = *reinterpret_cast<const v4i*>(xb + rt * 4096 + h * 2048 + 1024 + lane * 16);
-        xf[t] = v8i{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
-      }
-    }
+  for (int h = 0; h < 2; ++h)
 #pragma unroll
     for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
       for (int tm = 0; tm < 2; ++tm) {
         if (h == 0)
-          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[tn], xf[tm], acc[tn][tm], kFmtE2M1, FMT, 0,
-                                                                        scw[tn], 0, scx[tm]);
+          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(widen(wf[0][tn]), widen(xf[0][tm]), acc[tn][tm],
+                                                                        kFmtE2M1, FMT, 0, scw[tn], 0, scx[tm]);
         else
-          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[tn], xf[tm], acc[tn][tm], kFmtE2M1, FMT, 2,
-                                                                        scw[tn], 2, scx[tm]);
+          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(widen(wf[1][tn]), widen(xf[1][tm]), acc[tn][tm],
+                                                                        kFmtE2M1, FMT, 2, scw[tn], 2, scx[tm]);
       }
-  }
 }
 
-// Runs the stages of one segment.  On entry the staging registers hold stage 0 of
-// this segment; on exit they hold stage 0 of the next segment (if any).
+// Runs the stages of one segment.  While stage q is computed from one LDS buffer the copies
+// of stage q+1 (of this segment, or stage 0 of the next one) fill the other.  `pos` counts
+// stages across segments; LDS buffer = pos & 1.
 template <int FMT, int FMT_NEXT>
-__device__ __forceinline__ void segment_tiled(v16f (&acc)[4][2], Staging& st, const Seg& sg, const Seg& next,
-                                              uint8_t* __restrict__ lds, int& parity, int n0, int m0, int tid, int lane,
-                                              int wn, int wm) {
-  for (int q = 0; q < sg.stages; ++q) {
-    uint8_t* buf = lds + parity * kStageBytes;
-    stage_store<FMT>(st, buf, tid);
-    const v4i sw = st.sw, sx = st.sx;
-    if (q + 1 < sg.stages)
-      stage_load<FMT>(st, sg, q + 1, n0, m0, tid, lane, wn, wm);
-    else if (next.stages > 0)
-      stage_load<FMT_NEXT>(st, next, 0, n0, m0, tid, lane, wn, wm);
+__device__ __forceinline__ void segment_tiled(v16f (&acc)[4][2], const Seg& sg, const Seg& next, uint8_t* __restrict__ lds,
+                                              int& pos, int n0, int m0, int lane, int wave, int wn, int wm) {
+  if (sg.stages == 0) return;
+  const CopyOffsets<FMT> off(sg, lane);
+  for (int q = 0; q < sg.stages; ++q, ++pos) {
+    uint8_t* cur = lds + (pos & 1) * kStageBytes;
+    uint8_t* nxt = lds + ((pos + 1) & 1) * kStageBytes;
+    // this wave's copies for the current stage have landed; after the barrier everybody's have,
+    // and nobody still reads the other buffer
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     __syncthreads();
-    stage_compute<FMT>(acc, buf, sw, sx, lane, wn, wm);
-    parity ^= 1;
+    v4i wf[2][4], sw, sx;
+    typename XFrag<FMT>::type xf[2][2];
+    frags_read<FMT>(wf, xf, sw, sx, cur, lane, wn, wm);
+    if (q + 1 < sg.stages) {
+      stage_copy<FMT>(sg, off, q + 1, n0, m0, nxt, wave, lane);
+    } else if (next.stages > 0) {
+      const CopyOffsets<FMT_NEXT> noff(next, lane);
+      stage_copy<FMT_NEXT>(next, noff, 0, n0, m0, nxt, wave, lane);
+    }
+    stage_compute<FMT>(acc, wf, xf, sw, sx, lane, wm);
   }
 }
 
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 mixed_gemm_tiled_kernel(Seg s4, Seg s6, Seg s8, int M, int N, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
   const int n0 = blockIdx.x * kTileN, m0 = blockIdx.y * kTileM;
 
@@ -348,18 +366,19 @@ mixed_gemm_tiled_kernel(Seg s4, Seg s6, Seg s8, int M, int N, uint16_t* __restri
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
 
-  Staging st;
-  int parity = 0;
+  int pos = 0;
   const Seg none = {nullptr, nullptr, nullptr, nullptr, 0};
-  // prime the staging registers with the first stage of the first non-empty segment
-  if (s4.stages > 0) stage_load<kFmtE2M1>(st, s4, 0, n0, m0, tid, lane, wn, wm);
-  else if (s6.stages > 0) stage_load<kFmtE3M2>(st, s6, 0, n0, m0, tid, lane, wn, wm);
-  else if (s8.stages > 0) stage_load<kFmtE4M3>(st, s8, 0, n0, m0, tid, lane, wn, wm);
+  // an empty middle segment is skipped by handing its successor to the one before it
+  const Seg& after4 = s6.stages > 0 ? s6 : s8;
+  // first stage of the first non-empty segment
+  if (s4.stages > 0) stage_copy<kFmtE2M1>(s4, CopyOffsets<kFmtE2M1>(s4, lane), 0, n0, m0, lds, wave, lane);
+  else if (s6.stages > 0) stage_copy<kFmtE3M2>(s6, CopyOffsets<kFmtE3M2>(s6, lane), 0, n0, m0, lds, wave, lane);
+  else stage_copy<kFmtE4M3>(s8, CopyOffsets<kFmtE4M3>(s8, lane), 0, n0, m0, lds, wave, lane);
 
-  if (s6.stages > 0) segment_tiled<kFmtE2M1, kFmtE3M2>(acc, st, s4, s6, lds, parity, n0, m0, tid, lane, wn, wm);
-  else               segment_tiled<kFmtE2M1, kFmtE4M3>(acc, st, s4, s8, lds, parity, n0, m0, tid, lane, wn, wm);
-  segment_tiled<kFmtE3M2, kFmtE4M3>(acc, st, s6, s8, lds, parity, n0, m0, tid, lane, wn, wm);
-  segment_tiled<kFmtE4M3, kFmtE4M3>(acc, st, s8, none, lds, parity, n0, m0, tid, lane, wn, wm);
+  if (s6.stages > 0) segment_tiled<kFmtE2M1, kFmtE3M2>(acc, s4, after4, lds, pos, n0, m0, lane, wave, wn, wm);
+  else               segment_tiled<kFmtE2M1, kFmtE4M3>(acc, s4, after4, lds, pos, n0, m0, lane, wave, wn, wm);
+  segment_tiled<kFmtE3M2, kFmtE4M3>(acc, s6, s8, lds, pos, n0, m0, lane, wave, wn, wm);
+  segment_tiled<kFmtE4M3, kFmtE4M3>(acc, s8, none, lds, pos, n0, m0, lane, wave, wn, wm);
 
   // result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4
   const int g = lane >> 5;
@@ -373,6 +392,9 @@ mixed_gemm_tiled_kernel(Seg s4, Seg s6, Seg s8, int M, int N, uint16_t* __restri
       for (int vq = 0; vq < 4; ++vq) {
         const v2bf lo = {(__bf16)acc[tn][tm][4 * vq + 0], (__bf16)acc[tn][tm][4 * vq + 1]};
         const v2bf hi = {(__bf16)acc[tn][tm][4 * vq + 2], (__bf16)acc[tn][tm][4 * vq + 3]};
+#ifdef MG_EXP_NOSTORE
+        if (acc[tn][tm][4 * vq] == 12345.678f)
+#endif
         *reinterpret_cast<v2u*>(row + tn * 32 + vq * 8) =
             v2u{__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
       }

@@ -26,12 +26,11 @@ __device__ __forceinline__ unsigned perm(unsigned hi, unsigned lo, unsigned sel)
 // E8M0 byte of the block scale from the bits of amax (a non-negative float).
 // MAX = fm * 2^pm with fm in [0.5,1): the exponent steps up by one when the
 // mantissa of amax exceeds the mantissa of MAX, which the add below carries
-// into the exponent field.
-template <int FMT>
-__device__ __forceinline__ int scale_byte(float amax) {
-  constexpr unsigned thr = (FMT == kFmtE2M1) ? 0x400000u : 0x600000u;  // 6 = 1.5*4, 28 = 1.75*16, 448 = 1.75*256
-  constexpr int pm = (FMT == kFmtE2M1) ? 3 : (FMT == kFmtE3M2 ? 5 : 9);
-  unsigned bits = __float_as_uint(amax);
+// into the exponent field.  `fmt` may differ between the lanes of a wave.
+__device__ __forceinline__ int scale_byte(float amax, int fmt) {
+  const unsigned thr = fmt == kFmtE2M1 ? 0x400000u : 0x600000u;  // 6 = 1.5*4, 28 = 1.75*16, 448 = 1.75*256
+  const int pm = fmt == kFmtE2M1 ? 3 : (fmt == kFmtE3M2 ? 5 : 9);
+  const unsigned bits = __float_as_uint(amax);
   int byte = (int)((bits + (0x7FFFFFu - thr)) >> 23) + 1 - pm;
   byte = byte < 0 ? 0 : byte;
   return amax == 0.0f ? 126 : byte;
@@ -43,19 +42,24 @@ __device__ __forceinline__ float round_scaled(float x, float rs) {
   return __builtin_truncf(__builtin_fmaf(x, rs, half));
 }
 
-// Quantize one gathered block (32 floats holding bf16 values) into packed codes.
-template <int FMT>
-__device__ __forceinline__ int quantize_block(const float (&f)[32], unsigned (&out)[8]) {
+// Quantize one gathered block (32 floats holding bf16 values) and store its codes and scale.
+// Everything up to the integer-valued v[] is the same instruction stream for the three
+// formats (a wave that straddles a segment boundary runs it once, not once per format); only
+// the final conversion and store differ.
+__device__ __forceinline__ void quantize_store(const float (&f)[32], int fmt, uint8_t* __restrict__ q,
+                                               uint8_t* __restrict__ sf) {
   float amax = 0.0f;
 #pragma unroll
   for (int p = 0; p < 32; p += 2) amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(f[p]), __builtin_fabsf(f[p + 1])));
-  const int byte = scale_byte<FMT>(amax);
+  const int byte = scale_byte(amax, fmt);
   const float rs = __uint_as_float((unsigned)(254 - byte) << 23);
   float v[32];
 #pragma unroll
   for (int p = 0; p < 32; ++p) v[p] = round_scaled(f[p], rs);
+  *sf = (uint8_t)byte;
 
-  if constexpr (FMT == kFmtE2M1) {
+  if (fmt == kFmtE2M1) {
+    v4u out;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       unsigned w = 0;
@@ -65,51 +69,40 @@ __device__ __forceinline__ int quantize_block(const float (&f)[32], unsigned (&o
       w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, v[8 * j + 6], v[8 * j + 7], 1.0f, 3);
       out[j] = w;
     }
-  } else if constexpr (FMT == kFmtE3M2) {
+    *reinterpret_cast<v4u*>(q) = out;
+  } else {
+    // the bf16 hop of the reference (src/reorder.cu:223) is a real rounding above 256
     v32bf h;
 #pragma unroll
     for (int p = 0; p < 32; ++p) h[p] = (__bf16)v[p];
-    // the ISA calls E3M2 "bf6" (its "fp6" is E2M3)
-    v6u w = __builtin_amdgcn_cvt_scalef32_pk32_bf6_bf16(h, 1.0f);
+    if (fmt == kFmtE3M2) {
+      // the ISA calls E3M2 "bf6" (its "fp6" is E2M3)
+      const v6u w = __builtin_amdgcn_cvt_scalef32_pk32_bf6_bf16(h, 1.0f);
+      v2u* p = reinterpret_cast<v2u*>(q);
+      p[0] = v2u{w[0], w[1]};
+      p[1] = v2u{w[2], w[3]};
+      p[2] = v2u{w[4], w[5]};
+    } else {
+      unsigned out[8];
 #pragma unroll
-    for (int j = 0; j < 6; ++j) out[j] = w[j];
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      // the bf16 hop of the reference (src/reorder.cu:223) is a real rounding above 256
-      v2bf lo = {(__bf16)v[4 * j + 0], (__bf16)v[4 * j + 1]};
-      v2bf hi = {(__bf16)v[4 * j + 2], (__bf16)v[4 * j + 3]};
-      v2s z = {0, 0};
-      z = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(z, lo, 1.0f, false);
-      z = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(z, hi, 1.0f, true);
-      out[j] = __builtin_bit_cast(unsigned, z);
+      for (int j = 0; j < 8; ++j) {
+        const v2bf lo = {h[4 * j + 0], h[4 * j + 1]};
+        const v2bf hi = {h[4 * j + 2], h[4 * j + 3]};
+        v2s z = {0, 0};
+        z = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(z, lo, 1.0f, false);
+        z = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(z, hi, 1.0f, true);
+        out[j] = __builtin_bit_cast(unsigned, z);
+      }
+      v4u* p = reinterpret_cast<v4u*>(q);
+      p[0] = v4u{out[0], out[1], out[2], out[3]};
+      p[1] = v4u{out[4], out[5], out[6], out[7]};
     }
   }
-  return byte;
 }
 
-template <int FMT>
-__device__ __forceinline__ void quantize_store(const float (&f)[32], uint8_t* __restrict__ q, uint8_t* __restrict__ sf) {
-  unsigned out[8];
-  const int byte = quantize_block<FMT>(f, out);
-  if constexpr (FMT == kFmtE2M1) {
-    *reinterpret_cast<v4u*>(q) = v4u{out[0], out[1], out[2], out[3]};
-  } else if constexpr (FMT == kFmtE3M2) {
-    v2u* p = reinterpret_cast<v2u*>(q);
-    p[0] = v2u{out[0], out[1]};
-    p[1] = v2u{out[2], out[3]};
-    p[2] = v2u{out[4], out[5]};
-  } else {
-    v4u* p = reinterpret_cast<v4u*>(q);
-    p[0] = v4u{out[0], out[1], out[2], out[3]};
-    p[1] = v4u{out[4], out[5], out[6], out[7]};
-  }
-  *sf = (uint8_t)byte;
-}
-
-// One workgroup handles R consecutive rows; blockDim.x >= K/32.
-template <int R, bool IS_W>
-__global__ void __launch_bounds__(1024)
+// One workgroup handles R consecutive rows; blockDim.x >= K/32 (at most MAXT).
+template <int R, bool IS_W, int MAXT>
+__global__ void __launch_bounds__(MAXT)
 reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__ idx, int rows, int K, int KN, int KS,
                      int KO, uint8_t* __restrict__ qn, uint8_t* __restrict__ qs, uint8_t* __restrict__ qo,
                      uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo) {
@@ -118,40 +111,55 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
   const int nthr = blockDim.x;
   const int row0 = blockIdx.x * R;
 
-  // ---- stage R rows: coalesced 16-byte loads, R x 8 transpose in registers,
-  //      16-byte LDS stores.  Channel c of row r lands at lds[(c*R + r)*2].
+  // ---- the lane's 32 reorder indices: requested first, needed only after the barrier
+  const int b = tid;
+  const bool has_block = b < (K >> 5);
+  v4u iv[4];
+  {
+    const v4u* ip = reinterpret_cast<const v4u*>(idx + (size_t)(has_block ? b : 0) * 32);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) iv[q] = ip[q];
+  }
+
+  // ---- stage R rows: all 16-byte loads issued up front (row and chunk clamped instead of
+  //      branched, so nothing waits), R x 8 transpose in registers, 16-byte LDS stores.
+  //      Channel c of row r lands at lds[(c*R + r)*2].
   const int nchunks = K >> 3;
+  v4u a[4][R];
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int c = min(tid + it * nthr, nchunks - 1);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int row = min(row0 + r, rows - 1);
+      a[it][r] = *reinterpret_cast<const v4u*>(x + (size_t)row * K + (size_t)c * 8);
+    }
+  }
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const int c = tid + it * nthr;
     if (c < nchunks) {
-      v4u a[R];
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        a[r] = v4u{0, 0, 0, 0};
-        if (row0 + r < rows) a[r] = *reinterpret_cast<const v4u*>(x + (size_t)(row0 + r) * K + (size_t)c * 8);
-      }
       v4u* dst = reinterpret_cast<v4u*>(lds + (size_t)c * 16 * R);
       if constexpr (R == 1) {
-        dst[0] = a[0];
+        dst[0] = a[it][0];
       } else if constexpr (R == 2) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           v4u o;
-          o[0] = perm(a[1][2 * h], a[0][2 * h], 0x05040100u);
-          o[1] = perm(a[1][2 * h], a[0][2 * h], 0x07060302u);
-          o[2] = perm(a[1][2 * h + 1], a[0][2 * h + 1], 0x05040100u);
-          o[3] = perm(a[1][2 * h + 1], a[0][2 * h + 1], 0x07060302u);
+          o[0] = perm(a[it][1][2 * h], a[it][0][2 * h], 0x05040100u);
+          o[1] = perm(a[it][1][2 * h], a[it][0][2 * h], 0x07060302u);
+          o[2] = perm(a[it][1][2 * h + 1], a[it][0][2 * h + 1], 0x05040100u);
+          o[3] = perm(a[it][1][2 * h + 1], a[it][0][2 * h + 1], 0x07060302u);
           dst[h] = o;
         }
       } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           v4u o;
-          o[0] = perm(a[1][j], a[0][j], 0x05040100u);
-          o[1] = perm(a[3][j], a[2][j], 0x05040100u);
-          o[2] = perm(a[1][j], a[0][j], 0x07060302u);
-          o[3] = perm(a[3][j], a[2][j], 0x07060302u);
+          o[0] = perm(a[it][1][j], a[it][0][j], 0x05040100u);
+          o[1] = perm(a[it][3][j], a[it][2][j], 0x05040100u);
+          o[2] = perm(a[it][1][j], a[it][0][j], 0x07060302u);
+          o[3] = perm(a[it][3][j], a[it][2][j], 0x07060302u);
           dst[j] = o;
         }
       }
@@ -160,23 +168,25 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
   __syncthreads();
 
   // ---- one lane per 32-element block
-  const int b = tid;
-  if (b >= (K >> 5)) return;
+  if (!has_block) return;
   const int nbn = KN >> 5, nbs = KS >> 5;
   const int seg = b < nbn ? 0 : (b < nbn + nbs ? 1 : 2);
   const int j = seg == 0 ? b : (seg == 1 ? b - nbn : b - nbn - nbs);
   const int kseg = seg == 0 ? KN : (seg == 1 ? KS : KO);
   const int katoms = (kseg + 127) >> 7;
+  const int fmt = IS_W ? kFmtE2M1 : (seg == 0 ? kFmtE2M1 : (seg == 1 ? kFmtE3M2 : kFmtE4M3));
+  const int blk_bytes = fmt == kFmtE2M1 ? 16 : (fmt == kFmtE3M2 ? 24 : 32);
+  const size_t pitch = (size_t)(kseg >> 5) * blk_bytes;
+  uint8_t* qbase = (seg == 0 ? qn : (seg == 1 ? qs : qo)) + j * blk_bytes;
+  uint8_t* sfbase = seg == 0 ? sfn : (seg == 1 ? sfs : sfo);
 
   unsigned g[32][(R + 1) / 2];
   {
-    const v4u* ip = reinterpret_cast<const v4u*>(idx + (size_t)b * 32);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const v4u iv = ip[q];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const unsigned ch = (e & 1) ? (iv[e >> 1] >> 16) : (iv[e >> 1] & 0xffffu);
+        const unsigned ch = (e & 1) ? (iv[q][e >> 1] >> 16) : (iv[q][e >> 1] & 0xffffu);
         const int p = q * 8 + e;
         if constexpr (R == 4) {
           const v2u d = *reinterpret_cast<const v2u*>(lds + ch * 8);
@@ -201,19 +211,8 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
       const unsigned d = g[p][r >> 1];
       f[p] = __uint_as_float((r & 1) ? (d & 0xffff0000u) : (d << 16));
     }
-    if (seg == 0) {
-      quantize_store<kFmtE2M1>(f, qn + (size_t)row * (KN >> 1) + j * 16, sfn + sf_offset(row, j, katoms));
-    } else if (seg == 1) {
-      if constexpr (IS_W)
-        quantize_store<kFmtE2M1>(f, qs + (size_t)row * (KS >> 1) + j * 16, sfs + sf_offset(row, j, katoms));
-      else
-        quantize_store<kFmtE3M2>(f, qs + (size_t)row * (KS / 4 * 3) + j * 24, sfs + sf_offset(row, j, katoms));
-    } else {
-      if constexpr (IS_W)
-        quantize_store<kFmtE2M1>(f, qo + (size_t)row * (KO >> 1) + j * 16, sfo + sf_offset(row, j, katoms));
-      else
-        quantize_store<kFmtE4M3>(f, qo + (size_t)row * KO + j * 32, sfo + sf_offset(row, j, katoms));
-    }
+    // per-lane format, code row pitch and byte offset of the block inside its row
+    quantize_store(f, fmt, qbase + (size_t)row * pitch, sfbase + sf_offset(row, j, katoms));
   }
 }
 
@@ -227,15 +226,19 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
   const int threads = ((K >> 5) + 63) & ~63;
   const uint16_t* xb = static_cast<const uint16_t*>(x);
   // R rows interleaved in LDS; keep the tile within 64 KB so several workgroups share a CU
+#ifndef MG_QUANT_R_SMALLK
+#define MG_QUANT_R_SMALLK 2
+#endif
   if (K <= 8192) {
-    hipLaunchKernelGGL((reorder_quant_kernel<4, IS_W>), dim3(ceil_div(rows, 4)), dim3(threads), (size_t)K * 8, stream, xb,
-                       idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+    constexpr int R = MG_QUANT_R_SMALLK;
+    hipLaunchKernelGGL((reorder_quant_kernel<R, IS_W, 256>), dim3(ceil_div(rows, R)), dim3(threads), (size_t)K * 2 * R,
+                       stream, xb, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
   } else if (K <= 16384) {
-    hipLaunchKernelGGL((reorder_quant_kernel<2, IS_W>), dim3(ceil_div(rows, 2)), dim3(threads), (size_t)K * 4, stream, xb,
-                       idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+    hipLaunchKernelGGL((reorder_quant_kernel<2, IS_W, 512>), dim3(ceil_div(rows, 2)), dim3(threads), (size_t)K * 4, stream,
+                       xb, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
   } else {
-    hipLaunchKernelGGL((reorder_quant_kernel<1, IS_W>), dim3(rows), dim3(threads), (size_t)K * 2, stream, xb, idx, rows, K,
-                       KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+    hipLaunchKernelGGL((reorder_quant_kernel<1, IS_W, 1024>), dim3(rows), dim3(threads), (size_t)K * 2, stream, xb, idx,
+                       rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
   }
   return hipGetLastError();
 }

@@ -161,6 +161,8 @@ GEMM_SHAPES = [
     # whole 128 x 256 tiles and 128-wide K stages: the LDS-tiled kernel
     (128, 256, 256, 0, 0), (128, 256, 0, 256, 0), (128, 256, 0, 0, 128), (128, 256, 128, 0, 128),
     (256, 512, 384, 256, 128), (128, 256, 2560, 1408, 128), (384, 768, 1280, 640, 128),
+    # whole 256 x 256 tiles with all three segments: the one-workgroup-per-CU kernel
+    (256, 256, 128, 128, 128), (512, 256, 256, 384, 128), (256, 768, 2560, 1408, 128), (512, 512, 640, 256, 256),
 ]
 
 

@@ -134,6 +134,133 @@ mixed_gemm_direct_kernel(const uint8_t* __restrict__ an, const uint8_t* __restri
 
 
 // ---------------------------------------------------------------------------
+// Decode kernel: M <= 16 tokens, weights streamed once (HBM-bound).
+//
+// A workgroup of 4 waves owns 16 output features; the K steps (128 elements
+// each, counted over the three segments) are dealt to the 4 waves in contiguous
+// quarters, so 3.5 waves per SIMD each keep all their weight loads in flight at
+// once.  Every load of a wave is issued before its first MFMA; the 4 partial
+// 16x16 tiles are summed through LDS and rounded to bf16 once.
+// ---------------------------------------------------------------------------
+constexpr int kDecodeMaxSteps = 8;   // K steps a wave keeps in flight at once
+
+struct DecodeSeg {
+  const uint8_t* a;
+  const uint8_t* b;
+  const uint8_t* sfa;
+  const uint8_t* sfb;
+  int nblk;    // 32-element blocks in the segment
+  int steps;   // ceil(nblk / 4)
+};
+
+template <int FMT>
+__device__ __forceinline__ v4f decode_mfma(v8i wb, v8i xa, v4f acc, int sw, int sx) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wb, xa, acc, kFmtE2M1, FMT, 0, sw, 0, sx);
+}
+
+__global__ void __launch_bounds__(256)
+mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N, int steps_per_wave,
+                         uint16_t* __restrict__ d) {
+  __shared__ float partial[4][16 * 16];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i = lane & 15, g = lane >> 4;
+  const int n = blockIdx.x * 16 + i;
+  const bool n_ok = n < N, m_ok = i < M;
+  const int nc = min(n, N - 1), mc = min(i, M - 1);   // clamped rows: every load is in bounds and unconditional
+  const int total = s4.steps + s6.steps + s8.steps;
+  v4f acc = {0.f, 0.f, 0.f, 0.f};
+
+  for (int r0 = 0; r0 < steps_per_wave; r0 += kDecodeMaxSteps) {
+  const int t0 = wave * steps_per_wave + r0, t_end = min(total, wave * steps_per_wave + steps_per_wave);
+
+  // Straight-line issue of every load of this wave (addresses clamped, no
+  // branches), so all of them are in flight together; masking comes afterwards.
+  v4i wq[kDecodeMaxSteps], xa[kDecodeMaxSteps], xb[kDecodeMaxSteps];
+  int sw[kDecodeMaxSteps], sx[kDecodeMaxSteps];
+#pragma unroll
+  for (int k = 0; k < kDecodeMaxSteps; ++k) {
+    const int t = min(t0 + k, total - 1);
+    const int seg = t < s4.steps ? 0 : (t < s4.steps + s6.steps ? 1 : 2);
+    const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
+    const uint8_t* pa = seg == 0 ? s4.a : (seg == 1 ? s6.a : s8.a);
+    const uint8_t* pb = seg == 0 ? s4.b : (seg == 1 ? s6.b : s8.b);
+    const uint8_t* psa = seg == 0 ? s4.sfa : (seg == 1 ? s6.sfa : s8.sfa);
+    const uint8_t* psb = seg == 0 ? s4.sfb : (seg == 1 ? s6.sfb : s8.sfb);
+    const int nblk = seg == 0 ? s4.nblk : (seg == 1 ? s6.nblk : s8.nblk);
+    const int katoms = seg == 0 ? s4.steps : (seg == 1 ? s6.steps : s8.steps);
+    const int xbytes = seg == 0 ? 16 : (seg == 1 ? 24 : 32);   // activation bytes per 32-element block
+    const int left = nblk - 4 * q;
+    const int gc = min(g, left - 1);
+    wq[k] = *reinterpret_cast<const v4i*>(pb + (size_t)nc * nblk * 16 + q * 64 + gc * 16);
+    // activations: two 16-byte pieces.  E2M1: block g (second piece unused);
+    // E3M2: bytes [0,16) and [8,24) of block g; E4M3: K [16g,+16) and [64+16g,+16).
+    const uint8_t* xrow = pa + (size_t)mc * nblk * xbytes + q * 4 * xbytes;
+    const int a_blk = seg == 2 ? (g >> 1) : g, b_blk = seg == 2 ? 2 + (g >> 1) : g;
+    int off_a = seg == 1 ? g * 24 : g * 16;
+    int off_b = seg == 0 ? g * 16 : (seg == 1 ? g * 24 + 8 : 64 + g * 16);
+    off_a = a_blk < left ? off_a : 0;
+    off_b = b_blk < left ? off_b : 0;
+    xa[k] = *reinterpret_cast<const v4i*>(xrow + off_a);
+    xb[k] = *reinterpret_cast<const v4i*>(xrow + off_b);
+    sw[k] = psb[sf_offset(nc, 4 * q + gc, katoms)];
+    sx[k] = psa[sf_offset(mc, 4 * q + gc, katoms)];
+  }
+
+#pragma unroll
+  for (int k = 0; k < kDecodeMaxSteps; ++k) {
+    const int t = t0 + k;
+    if (t < t_end) {   // wave-uniform
+      const int seg = t < s4.steps ? 0 : (t < s4.steps + s6.steps ? 1 : 2);
+      const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
+      const int nblk = seg == 0 ? s4.nblk : (seg == 1 ? s6.nblk : s8.nblk);
+      const int left = nblk - 4 * q;
+      const bool blk_ok = g < left;
+      const bool w_ok = n_ok && blk_ok;
+      const v4i z = {0, 0, 0, 0};
+      const v4i w4 = w_ok ? wq[k] : z;
+      const v8i wf = {w4[0], w4[1], w4[2], w4[3], 0, 0, 0, 0};
+      const int s_w = w_ok ? sw[k] : 127;
+      const int s_x = (m_ok && blk_ok) ? sx[k] : 127;
+      if (seg == 0) {
+        const v4i a4 = (m_ok && blk_ok) ? xa[k] : z;
+        const v8i xf = {a4[0], a4[1], a4[2], a4[3], 0, 0, 0, 0};
+        acc = decode_mfma<kFmtE2M1>(wf, xf, acc, s_w, s_x);
+      } else if (seg == 1) {
+        const v4i a4 = (m_ok && blk_ok) ? xa[k] : z;
+        const v4i b4 = (m_ok && blk_ok) ? xb[k] : z;
+        const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4[2], b4[3], 0, 0};
+        acc = decode_mfma<kFmtE3M2>(wf, xf, acc, s_w, s_x);
+      } else {
+        const v4i a4 = (m_ok && (g >> 1) < left) ? xa[k] : z;
+        const v4i b4 = (m_ok && 2 + (g >> 1) < left) ? xb[k] : z;
+        const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4[0], b4[1], b4[2], b4[3]};
+        acc = decode_mfma<kFmtE4M3>(wf, xf, acc, s_w, s_x);
+      }
+    }
+  }
+  }
+
+  // result tile is D^T: lane holds token m = lane % 16, features 4 * (lane / 16) + v
+  *reinterpret_cast<v4f*>(&partial[wave][lane * 4]) = acc;
+  __syncthreads();
+  if (wave == 0) {
+    v4f sum = acc;
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const v4f p = *reinterpret_cast<const v4f*>(&partial[w][lane * 4]);
+      sum += p;
+    }
+    const int nn = blockIdx.x * 16 + 4 * g;
+    if (m_ok) {
+      uint16_t* dst = d + (size_t)i * N + nn;
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        if (nn + v < N) dst[v] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // LDS-tiled kernel on v_mfma_scale_f32_32x32x64_f8f6f4.
 //
 // Geometry of that instruction (measured on gfx950): lane l supplies row
@@ -392,9 +519,6 @@ mixed_gemm_tiled_kernel(Seg s4, Seg s6, Seg s8, int M, int N, uint16_t* __restri
       for (int vq = 0; vq < 4; ++vq) {
         const v2bf lo = {(__bf16)acc[tn][tm][4 * vq + 0], (__bf16)acc[tn][tm][4 * vq + 1]};
         const v2bf hi = {(__bf16)acc[tn][tm][4 * vq + 2], (__bf16)acc[tn][tm][4 * vq + 3]};
-#ifdef MG_EXP_NOSTORE
-        if (acc[tn][tm][4 * vq] == 12345.678f)
-#endif
         *reinterpret_cast<v2u*>(row + tn * 32 + vq * 8) =
             v2u{__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
       }
@@ -408,6 +532,15 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
                              int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
   if (M == 0 || N == 0) return hipSuccess;
+  if (M <= 16) {
+    const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
+    const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
+    const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};
+    const int steps_per_wave = (d4.steps + d6.steps + d8.steps + 3) / 4;
+    hipLaunchKernelGGL(mixed_gemm_decode_kernel, dim3(ceil_div(N, 16)), dim3(256), 0, stream, d4, d6, d8, M, N,
+                       steps_per_wave, static_cast<uint16_t*>(d));
+    return hipGetLastError();
+  }
   // the tiled kernel needs whole tiles and whole 128-wide K stages
   if (M % kTileM == 0 && N % kTileN == 0 && KN % kStageK == 0 && KS % kStageK == 0 && KO % kStageK == 0 &&
       KN + KS + KO > 0) {

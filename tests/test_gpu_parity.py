@@ -158,6 +158,8 @@ GEMM_SHAPES = [
     (16, 64, 128, 128, 128), (8, 64, 256, 128, 128), (33, 80, 64, 96, 32),
     (64, 128, 512, 384, 128), (114, 256, 2560, 896, 128), (128, 512, 2560, 1408, 128),
     (20, 64, 448, 224, 64), (1, 16, 32, 32, 32),
+    # decode kernel (M <= 16): ragged N, partial K steps, more K steps than one pass keeps in flight
+    (8, 200, 96, 160, 64), (3, 1000, 2560, 1408, 128), (16, 48, 8192, 4096, 1024), (5, 40, 0, 4928, 448),
     # whole 128 x 256 tiles and 128-wide K stages: the LDS-tiled kernel
     (128, 256, 256, 0, 0), (128, 256, 0, 256, 0), (128, 256, 0, 0, 128), (128, 256, 128, 0, 128),
     (256, 512, 384, 256, 128), (128, 256, 2560, 1408, 128), (384, 768, 1280, 640, 128),

@@ -507,31 +507,60 @@ mixed_gemm_tiled_kernel(Seg s4, Seg s6, Seg s8, int M, int N, uint16_t* __restri
   segment_tiled<kFmtE3M2, kFmtE4M3>(acc, s6, s8, lds, pos, n0, m0, lane, wave, wn, wm);
   segment_tiled<kFmtE4M3, kFmtE4M3>(acc, s8, none, lds, pos, n0, m0, lane, wave, wn, wm);
 
-  // result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4
-  const int g = lane >> 5;
+  // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.
+  // Written straight from that layout a store instruction would touch 32 rows with 16 bytes each;
+  // instead each wave transposes its 64 tokens x 128 features through its own quarter of the (now
+  // idle) LDS, so that a store instruction writes 4 rows x 256 contiguous bytes.
+  constexpr int kPitch = 256 + 16;   // bytes per token row in LDS
+  static_assert(4 * 64 * kPitch <= 2 * kStageBytes, "epilogue staging must fit the stage buffers");
+  __syncthreads();                   // every wave is done with the last stage's fragments
+  uint8_t* stage = lds + wave * 64 * kPitch;
+  {
+    const int g = lane >> 5;
+    uint8_t* wr = stage + (lane & 31) * kPitch + 8 * g;
 #pragma unroll
-  for (int tm = 0; tm < 2; ++tm) {
-    const int m = m0 + wm * 64 + tm * 32 + (lane & 31);
-    uint16_t* row = d + (size_t)m * N + n0 + wn * 128 + 4 * g;
+    for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-    for (int tn = 0; tn < 4; ++tn)
+      for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
-      for (int vq = 0; vq < 4; ++vq) {
-        const v2bf lo = {(__bf16)acc[tn][tm][4 * vq + 0], (__bf16)acc[tn][tm][4 * vq + 1]};
-        const v2bf hi = {(__bf16)acc[tn][tm][4 * vq + 2], (__bf16)acc[tn][tm][4 * vq + 3]};
-        *reinterpret_cast<v2u*>(row + tn * 32 + vq * 8) =
-            v2u{__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
-      }
+        for (int vq = 0; vq < 4; ++vq) {
+          const v2bf lo = {(__bf16)acc[tn][tm][4 * vq + 0], (__bf16)acc[tn][tm][4 * vq + 1]};
+          const v2bf hi = {(__bf16)acc[tn][tm][4 * vq + 2], (__bf16)acc[tn][tm][4 * vq + 3]};
+          *reinterpret_cast<v2u*>(wr + tm * 32 * kPitch + tn * 64 + vq * 16) =
+              v2u{__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
+        }
+  }
+  // only this wave reads what it wrote: no workgroup barrier needed
+  {
+    const int r = lane >> 4, c = lane & 15;
+    const uint8_t* rd = stage + r * kPitch + c * 16;
+    uint16_t* out = d + (size_t)(m0 + wm * 64 + r) * N + n0 + wn * 128 + c * 8;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const v4u v = *reinterpret_cast<const v4u*>(rd + i * 4 * kPitch);
+      *reinterpret_cast<v4u*>(out + (size_t)i * 4 * N) = v;
+    }
   }
 }
 
 }  // namespace
 
+#ifdef MG_USE_256
+bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO);
+hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
+                                 const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
+                                 const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
+                                 int M, int N, int KN, int KS, int KO, void* d, hipStream_t stream);
+#endif
 hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
                              int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
   if (M == 0 || N == 0) return hipSuccess;
+#ifdef MG_USE_256
+  if (mixed_gemm_256_supported(M, N, KN, KS, KO))
+    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, N, KN, KS, KO, d, stream);
+#endif
   if (M <= 16) {
     const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
     const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};

@@ -545,22 +545,20 @@ mixed_gemm_tiled_kernel(Seg s4, Seg s6, Seg s8, int M, int N, uint16_t* __restri
 
 }  // namespace
 
-#ifdef MG_USE_256
+// 256 x 256 tiles, one workgroup per CU (mixed_gemm_256.hip)
 bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO);
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
                                  int M, int N, int KN, int KS, int KO, void* d, hipStream_t stream);
-#endif
+
 hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
                              int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
   if (M == 0 || N == 0) return hipSuccess;
-#ifdef MG_USE_256
   if (mixed_gemm_256_supported(M, N, KN, KS, KO))
     return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, N, KN, KS, KO, d, stream);
-#endif
   if (M <= 16) {
     const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
     const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};

@@ -1,0 +1,697 @@
+// Mixed block-scaled GEMM for large whole-tile shapes: 256 x 256 workgroup tiles, one workgroup
+// of 4 waves per CU, each wave 128 features x 128 tokens = 4 x 4 tiles of
+// v_mfma_scale_f32_32x32x64_f8f6f4 (256 accumulator registers).  Replaces the three CUTLASS GEMMs
+// of the reference (src/fp4.cu:35, src/fp6.cu:35, src/fp8.cu:35, driver src/gemm.cu:22-47) for
+// M, N multiples of 256 and every K segment a non-empty multiple of 128.
+//
+// With one wave per SIMD nothing hides a wave's own instruction issue: next to an MFMA (32 cycles
+// in the matrix pipe) a wave gets only a handful of other instructions for free, so the steady
+// state is written to need about two per MFMA:
+//   * operands and scale atoms go global -> LDS directly (global_load_lds_dwordx4); a copy is a
+//     scalar base (advanced once per stage), a per-lane offset fixed for the segment, and an LDS
+//     offset that is an immediate (the three stage buffers are three copies of the loop body);
+//   * fragment reads use per-lane LDS addresses fixed for the segment plus immediates;
+//   * copies are spread between the MFMAs (the address unit needs about two MFMA times for one
+//     copy of each of the four waves).
+// Pipeline per K stage q (128 elements), three LDS buffers:
+//   read second half of q | 16 MFMAs first half, last copies of q+2 | own reads done, own copies
+//   of q+1 landed (those of q+2 stay in flight) | barrier | read first half + scales of q+1 |
+//   16 MFMAs second half, first copies of q+3 into the buffer stage q just freed.
+// The last three stages of a segment copy stages of the next segment(s); they run a generic body
+// whose copy format is a run-time, wave-uniform value.
+// The result tile is transposed through LDS so that stores write 256 contiguous bytes per row.
+#include "mg_common.h"
+
+namespace mg {
+
+namespace {
+
+constexpr int kT = 256;                   // tile edge (features and tokens)
+constexpr int kBlk = 1040;                // 16 rows x 64 B + 16
+constexpr int kBlk6 = 3088;               // 32 rows x 96 B + 16
+constexpr int kWOff = 0;
+constexpr int kXOff = 16 * kBlk;          // 16640
+constexpr int kSOff = kXOff + 32 * kBlk;  // E4M3 worst case: two K halves x 16 blocks -> 49920
+constexpr int kStage = kSOff + 2048;      // 51968
+constexpr int kBuffers = 3;
+constexpr int kCopySlots = 13;            // 4 weight copies, up to 8 token copies, 1 scale copy per wave and stage
+constexpr int kSplit = 5;                 // slots [0, kSplit) go out in the second half of a stage, the rest in the next first half
+
+typedef int v6i __attribute__((ext_vector_type(6)));
+
+// Kernel arguments: per K segment (0: E2M1, 1: E3M2, 2: E4M3 activations) the code and scale
+// pointers and the number of 128-wide stages.
+struct Plan {
+  const uint8_t *a0, *a1, *a2;        // activation codes
+  const uint8_t *b0, *b1, *b2;        // weight codes
+  const uint8_t *sfa0, *sfa1, *sfa2;  // activation scales
+  const uint8_t *sfb0, *sfb1, *sfb2;  // weight scales
+  int st0, st1, st2;                  // stages per segment
+  int total;                          // stages over all segments
+};
+
+__device__ __forceinline__ const uint8_t* uni(const uint8_t* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return reinterpret_cast<const uint8_t*>(((uint64_t)hi << 32) | lo);
+}
+
+// Field of segment sg (0, 1, 2) by masking rather than by select: a select between adjacent struct
+// fields is rewritten by the compiler into a dynamically indexed load from a private copy.
+__device__ __forceinline__ uint64_t pick3(int sg, uint64_t v0, uint64_t v1, uint64_t v2) {
+  const uint64_t m0 = sg == 0 ? ~0ull : 0ull, m1 = sg == 1 ? ~0ull : 0ull, m2 = sg == 2 ? ~0ull : 0ull;
+  return (v0 & m0) | (v1 & m1) | (v2 & m2);
+}
+__device__ __forceinline__ const uint8_t* pick3(int sg, const uint8_t* p0, const uint8_t* p1, const uint8_t* p2) {
+  return reinterpret_cast<const uint8_t*>(pick3(sg, reinterpret_cast<uint64_t>(p0), reinterpret_cast<uint64_t>(p1),
+                                                reinterpret_cast<uint64_t>(p2)));
+}
+__device__ __forceinline__ unsigned pick3u(int sg, unsigned v0, unsigned v1, unsigned v2) {
+  const unsigned m0 = sg == 0 ? ~0u : 0u, m1 = sg == 1 ? ~0u : 0u, m2 = sg == 2 ? ~0u : 0u;
+  return (v0 & m0) | (v1 & m1) | (v2 & m2);
+}
+
+// Which segment a global stage index falls in (uniform).
+__device__ __forceinline__ int seg_of(const Plan& p, int q, int& local) {
+  if (q < p.st0) { local = q; return 0; }
+  q -= p.st0;
+  if (q < p.st1) { local = q; return 1; }
+  local = q - p.st1;
+  return 2;
+}
+
+template <int FMT> struct Fmt;
+template <> struct Fmt<kFmtE2M1> { static constexpr int seg = 0, row_bytes = 64, x_copies = 4; typedef v4i xfrag; };
+template <> struct Fmt<kFmtE3M2> { static constexpr int seg = 1, row_bytes = 96, x_copies = 6; typedef v6i xfrag; };
+template <> struct Fmt<kFmtE4M3> { static constexpr int seg = 2, row_bytes = 128, x_copies = 8; typedef v8i xfrag; };
+
+// ---------------------------------------------------------------------------------------------
+// Copies.  One instruction moves 64 x 16 B to 1 KB of consecutive LDS.  Weights and E2M1 / E4M3
+// tokens: 16 rows x 64 B (a lane quad reads 64 contiguous bytes of one row), rows j, j+16, ...,
+// j+240 of the tile into block j at j * 1040 (E4M3: one set of 16 blocks per 64-wide K half).
+// E3M2 rows are 96 B: three instructions move the 32 rows j, j+8, ..., j+248 as one row-major
+// block of 3072 B at j * 3088.  Slot 12: waves 0, 2 copy the two weight scale atoms of the stage,
+// waves 1, 3 the two token scale atoms (twice the same bytes to the same place, so that every
+// wave issues the same number of copies and waits with the same count).
+// ---------------------------------------------------------------------------------------------
+
+// global[base + voff(lane)] -> LDS[lds_off + 16 * lane]; base and lds_off are wave-uniform
+__device__ __forceinline__ void copy16(const uint8_t* base, unsigned voff, unsigned lds_off) {
+  base = uni(base);
+  lds_off = __builtin_amdgcn_readfirstlane(lds_off);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               : : "v"(voff), "s"(base), "s"(lds_off) : "memory", "m0");
+}
+
+// the same with the LDS offset as scalar register + immediate
+template <int OFF>
+__device__ __forceinline__ void copy16i(const uint8_t* base, unsigned voff, unsigned lds_sreg) {
+  asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               : : "v"(voff), "s"(base), "s"(lds_sreg), "n"(OFF) : "memory", "m0", "scc");
+}
+
+// Per-lane byte offsets of the copies, fixed for the whole kernel.
+struct LaneOffsets {
+  unsigned w0, w1, w2;      // 16 rows apart per lane quad, 64-byte rows of pitch ldb of segment 0 / 1 / 2 (also E2M1 tokens)
+  unsigned x8;              // E4M3 tokens: pitch lda of segment 2
+  unsigned x6a, x6b, x6c;   // E3M2 tokens: piece (64k + lane) % 6 of row 8 * ((64k + lane) / 6), k = 0, 1, 2
+  unsigned s0, s1, s2;      // scale atoms: lanes 0-31 the first 128 rows, 32-63 the next 128
+
+  __device__ __forceinline__ LaneOffsets(const Plan& p, int lane) {
+    // quad k of a copy holds tile row j + 16 * (2 * (k % 8) + k / 8): rows 32t + i and 32t + i + 16 of a
+    // fragment end up 512 B apart in their block, which the LDS reads conflict-free (64 B apart they collide)
+    const unsigned k = lane >> 2, pr = 2 * (k & 7) + (k >> 3), c = lane & 3;
+    w0 = 16 * pr * (p.st0 * 64) + c * 16;
+    w1 = 16 * pr * (p.st1 * 64) + c * 16;
+    w2 = 16 * pr * (p.st2 * 64) + c * 16;
+    x8 = 16 * pr * (p.st2 * 128) + c * 16;
+    const unsigned lda6 = p.st1 * 96, c0 = lane, c1 = 64 + lane, c2 = 128 + lane;
+    x6a = 8 * (c0 / 6) * lda6 + (c0 % 6) * 16;
+    x6b = 8 * (c1 / 6) * lda6 + (c1 % 6) * 16;
+    x6c = 8 * (c2 / 6) * lda6 + (c2 % 6) * 16;
+    const unsigned hi = lane >> 5, lo = (lane & 31) * 16;
+    s0 = hi * p.st0 * 512 + lo;
+    s1 = hi * p.st1 * 512 + lo;
+    s2 = hi * p.st2 * 512 + lo;
+  }
+};
+
+struct Ctx {
+  int n0, m0, lane, wave, wn, wm, total;
+  unsigned lds_base;   // LDS byte offset of the dynamic shared memory
+#ifdef MG_TICKS
+  uint64_t* ticks;
+#endif
+};
+
+// Wave-uniform bases of the copies of global stage q (any segment).
+struct StageBases {
+  const uint8_t *w, *x, *s;
+  unsigned ldb, lda;
+  int seg;   // -1: no such stage
+
+  __device__ __forceinline__ StageBases() : w(nullptr), x(nullptr), s(nullptr), ldb(0), lda(0), seg(-1) {}
+
+  __device__ __forceinline__ StageBases(const Plan& plan, int q, const Ctx& c) {
+    int ql;
+    const int sg = seg_of(plan, q, ql);
+    seg = q < plan.total ? sg : -1;
+    const uint8_t* pa = pick3(sg, plan.a0, plan.a1, plan.a2);
+    const uint8_t* pb = pick3(sg, plan.b0, plan.b1, plan.b2);
+    const uint8_t* psa = pick3(sg, plan.sfa0, plan.sfa1, plan.sfa2);
+    const uint8_t* psb = pick3(sg, plan.sfb0, plan.sfb1, plan.sfb2);
+    const unsigned nst = (unsigned)pick3(sg, (uint64_t)plan.st0, (uint64_t)plan.st1, (uint64_t)plan.st2);
+    const unsigned rb = sg == 0 ? 64 : (sg == 1 ? 96 : 128);
+    ldb = nst * 64;
+    lda = nst * rb;
+    w = pb + (size_t)(c.n0 + c.wave * 4) * ldb + (size_t)ql * 64;
+    // first token row of the wave: E2M1 4*wave (+kx), E3M2 2*wave (+kx/3), E4M3 8*(wave%2) (+kx) in K half wave/2
+    const unsigned xrow = sg == 0 ? c.wave * 4 : (sg == 1 ? c.wave * 2 : (c.wave & 1) * 8);
+    x = pa + (size_t)(c.m0 + xrow) * lda + (size_t)ql * rb + (sg == 2 ? (c.wave >> 1) * 64 : 0);
+    s = (c.wave & 1) == 0 ? psb + ((size_t)(c.n0 >> 7) * nst + ql) * 512 : psa + ((size_t)(c.m0 >> 7) * nst + ql) * 512;
+  }
+};
+
+// Copies of a stage whose format is only known at run time (segment boundaries, prologue).
+struct GenericCopy {
+  StageBases b;
+  unsigned buf;   // LDS byte offset of the target stage buffer
+
+  __device__ __forceinline__ GenericCopy() : buf(0) {}
+  __device__ __forceinline__ GenericCopy(const Plan& plan, int q, const Ctx& c)
+      : b(plan, q, c), buf(c.lds_base + (q % kBuffers) * kStage) {}
+
+  __device__ __forceinline__ int count() const {
+    return b.seg < 0 ? 0 : 4 + (b.seg == 0 ? 4 : (b.seg == 1 ? 6 : 8)) + 1;
+  }
+
+  template <int K>
+  __device__ __forceinline__ void issue(const LaneOffsets& lo, int wave) const {
+    if (b.seg < 0) return;
+    if constexpr (K < 4) {
+      copy16(b.w + (size_t)K * b.ldb, pick3u(b.seg, lo.w0, lo.w1, lo.w2), buf + kWOff + (wave * 4 + K) * kBlk);
+    } else if constexpr (K < 12) {
+      constexpr int kx = K - 4;
+      if (b.seg == 0) {
+        if constexpr (kx < 4) copy16(b.x + (size_t)kx * b.lda, lo.w0, buf + kXOff + (wave * 4 + kx) * kBlk);
+      } else if (b.seg == 1) {
+        if constexpr (kx < 6)
+          copy16(b.x + (size_t)(kx / 3) * b.lda, kx % 3 == 0 ? lo.x6a : (kx % 3 == 1 ? lo.x6b : lo.x6c),
+                 buf + kXOff + (wave * 2 + kx / 3) * kBlk6 + (kx % 3) * 1024);
+      } else {
+        copy16(b.x + (size_t)kx * b.lda, lo.x8, buf + kXOff + (wave * 8 + kx) * kBlk);
+      }
+    } else {
+      copy16(b.s, pick3u(b.seg, lo.s0, lo.s1, lo.s2), buf + kSOff + (wave & 1) * 1024);
+    }
+  }
+};
+
+template <int K0, int K1>
+__device__ __forceinline__ void issue_range(const GenericCopy& cp, const LaneOffsets& lo, int wave) {
+  if constexpr (K0 < K1) {
+    cp.template issue<K0>(lo, wave);
+    issue_range<K0 + 1, K1>(cp, lo, wave);
+  }
+}
+
+// Copies of stages inside one segment of format FMT: scalar bases advanced by one stage at a time,
+// per-lane offsets (one register per copy, the row step of the copy folded in) fixed.
+template <int FMT>
+struct LeanCopy {
+  static constexpr int NX = Fmt<FMT>::x_copies;
+  const uint8_t *w, *x, *s;        // bases of the stage being copied
+  unsigned lds_w, lds_x, lds_s;    // LDS offsets of the wave's first weight / token block and scale atom pair in buffer 0
+  unsigned vw[4], vx[NX], vs;
+
+  __device__ __forceinline__ void init(const Plan& plan, int q, const LaneOffsets& lo, const Ctx& c) {
+    const StageBases b(plan, q, c);
+    w = uni(b.w);
+    x = uni(b.x);
+    s = uni(b.s);
+    constexpr int sg = Fmt<FMT>::seg;
+    const unsigned w_off = sg == 0 ? lo.w0 : (sg == 1 ? lo.w1 : lo.w2);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) vw[k] = w_off + k * b.ldb;
+#pragma unroll
+    for (int k = 0; k < NX; ++k) {
+      if constexpr (FMT == kFmtE2M1) vx[k] = vw[k];
+      else if constexpr (FMT == kFmtE3M2) vx[k] = (k % 3 == 0 ? lo.x6a : (k % 3 == 1 ? lo.x6b : lo.x6c)) + (k / 3) * b.lda;
+      else vx[k] = lo.x8 + k * b.lda;
+    }
+    vs = sg == 0 ? lo.s0 : (sg == 1 ? lo.s1 : lo.s2);
+    lds_w = __builtin_amdgcn_readfirstlane(c.lds_base + kWOff + c.wave * 4 * kBlk);
+    lds_x = __builtin_amdgcn_readfirstlane(c.lds_base + kXOff +
+                                           c.wave * (FMT == kFmtE2M1 ? 4 * kBlk : (FMT == kFmtE3M2 ? 2 * kBlk6 : 8 * kBlk)));
+    lds_s = __builtin_amdgcn_readfirstlane(c.lds_base + kSOff + (c.wave & 1) * 1024);
+  }
+
+  __device__ __forceinline__ void advance() {
+    w += 64;
+    x += Fmt<FMT>::row_bytes;
+    s += 512;
+  }
+
+  static constexpr int count() { return 4 + NX + 1; }
+
+  // slot K into the stage buffer at byte offset boff (wave-uniform)
+  template <int K>
+  __device__ __forceinline__ void issue(unsigned boff) const {
+    if constexpr (K < 4) {
+      copy16i<K * kBlk>(w, vw[K], lds_w + boff);
+    } else if constexpr (K < 4 + NX) {
+      constexpr int kx = K - 4;
+      if constexpr (FMT == kFmtE3M2) copy16i<(kx / 3) * kBlk6 + (kx % 3) * 1024>(x, vx[kx], lds_x + boff);
+      else copy16i<kx * kBlk>(x, vx[kx], lds_x + boff);
+    } else if constexpr (K == 12) {
+      copy16i<0>(s, vs, lds_s + boff);
+    }
+  }
+};
+
+// s_waitcnt vmcnt(n) for a run-time, wave-uniform n: the n most recent copies may stay in flight
+__device__ __forceinline__ void wait_copies_but(int n) {
+  switch (n) {
+#define MG_VMCNT_CASE(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
+    MG_VMCNT_CASE(1) MG_VMCNT_CASE(2) MG_VMCNT_CASE(3) MG_VMCNT_CASE(4) MG_VMCNT_CASE(5) MG_VMCNT_CASE(6)
+    MG_VMCNT_CASE(7) MG_VMCNT_CASE(8) MG_VMCNT_CASE(9) MG_VMCNT_CASE(10) MG_VMCNT_CASE(11) MG_VMCNT_CASE(12)
+    MG_VMCNT_CASE(13) MG_VMCNT_CASE(14) MG_VMCNT_CASE(15) MG_VMCNT_CASE(16) MG_VMCNT_CASE(17) MG_VMCNT_CASE(18)
+    MG_VMCNT_CASE(19) MG_VMCNT_CASE(20)
+#undef MG_VMCNT_CASE
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+  }
+}
+template <int N>
+__device__ __forceinline__ void wait_copies_but_imm() {
+  static_assert(N >= 0 && N < 64, "vmcnt immediate");
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// s_waitcnt lgkmcnt(0) as a compiler-visible instruction (vmcnt and expcnt fields at their maxima),
+// so that the compiler's own wait insertion knows the LDS reads are done
+__device__ __forceinline__ void wait_lds_reads() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+
+// ---------------------------------------------------------------------------------------------
+// Fragments
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ v8i widen(v4i v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1); }
+__device__ __forceinline__ v8i widen(v6i v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3, 4, 5, -1, -1); }
+__device__ __forceinline__ v8i widen(v8i v) { return v; }
+
+// Fragments of one 64-wide K half of a stage: 4 feature tiles, 4 token tiles.
+template <int FMT>
+struct HalfFrags {
+  v4i w[4];
+  typename Fmt<FMT>::xfrag x[4];
+};
+
+// Per-lane LDS addresses of a wave's fragments in stage buffer 0.
+struct WeightPtrs {
+  const uint8_t* w;    // weights: row 32*t + i at block i%16, quad 8*(i/16) + t; + t*64 + h*32
+  const uint8_t* sw;   // scale dwords of the 4 feature tiles
+  const uint8_t* sx;   // scale dwords of the 4 token tiles
+
+  __device__ __forceinline__ WeightPtrs(const uint8_t* lds, const Ctx& c) {
+    const int i = c.lane & 31, g = c.lane >> 5;
+    w = lds + kWOff + (i & 15) * kBlk + (i >> 4) * 512 + c.wn * 256 + g * 16;
+    sw = lds + kSOff + c.wn * 512 + i * 16;
+    sx = lds + kSOff + 1024 + c.wm * 512 + i * 16;
+  }
+};
+
+template <int FMT>
+struct TokenPtrs {
+  const uint8_t* x;
+
+  __device__ __forceinline__ TokenPtrs(const uint8_t* lds, const Ctx& c) {
+    const int i = c.lane & 31, g = c.lane >> 5;
+    if constexpr (FMT == kFmtE3M2) {
+      // row 32*rt + i: block i%8, row slot 4*rt + i/8, fragment 2h+g of 24 bytes
+      x = lds + kXOff + (i & 7) * kBlk6 + (16 * c.wm + (i >> 3)) * 96 + g * 24;
+    } else {
+      x = lds + kXOff + (i & 15) * kBlk + (i >> 4) * 512 + c.wm * 256 + g * 16;
+    }
+  }
+};
+
+// Reads of the fragments of K half H of one stage, one fragment per call so that they can be
+// spread between MFMAs: R = 0..3 weight tile R, 4..7 token tile R-4, 8 / 9 the scale dwords of
+// the feature / token tiles (only when SC).
+template <int FMT, int H, bool SC>
+struct FragReader {
+  HalfFrags<FMT>& f;
+  v4i& sw;
+  v4i& sx;
+  const uint8_t* pw;
+  const uint8_t* px;
+  const uint8_t* psw;
+  const uint8_t* psx;
+  bool on;   // wave-uniform
+
+  static constexpr int kReads = SC ? 10 : 8;
+
+  template <int R>
+  __device__ __forceinline__ void read() const {
+    if (!on) return;
+    if constexpr (R < 4) {
+      f.w[R] = *reinterpret_cast<const v4i*>(pw + R * 64 + H * 32);
+    } else if constexpr (R < 8) {
+      constexpr int t = R - 4;
+      if constexpr (FMT == kFmtE2M1) {
+        f.x[t] = *reinterpret_cast<const v4i*>(px + t * 64 + H * 32);
+      } else if constexpr (FMT == kFmtE3M2) {
+        const v2i* p = reinterpret_cast<const v2i*>(px + t * 384 + H * 48);
+        const v2i a = p[0], b = p[1], c = p[2];
+        f.x[t] = v6i{a[0], a[1], b[0], b[1], c[0], c[1]};
+      } else {
+        const uint8_t* p = px + H * 16 * kBlk + t * 64;
+        const v4i a = *reinterpret_cast<const v4i*>(p);        // K [16g, 16g+16) of the half
+        const v4i b = *reinterpret_cast<const v4i*>(p + 32);   // K [32+16g, 32+16g+16)
+        f.x[t] = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+    } else if constexpr (SC && R == 8) {
+      sw = *reinterpret_cast<const v4i*>(psw);
+    } else if constexpr (SC && R == 9) {
+      sx = *reinterpret_cast<const v4i*>(psx);
+    }
+  }
+};
+
+template <int FMT, int H, bool SC, int R = 0>
+__device__ __forceinline__ void read_all(const FragReader<FMT, H, SC>& rd) {
+  if constexpr (R < FragReader<FMT, H, SC>::kReads) {
+    rd.template read<R>();
+    read_all<FMT, H, SC, R + 1>(rd);
+  }
+}
+
+struct Scales {
+  int w[4], x[4];   // scale dwords of the 4 feature / 4 token tiles, shifted so that byte 0 / 2 is block g / 2+g
+};
+
+__device__ __forceinline__ void shift_scales(Scales& sc, v4i sw, v4i sx, int lane) {
+  const int g8 = (lane >> 5) * 8;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    sc.w[t] = (int)((unsigned)sw[t] >> g8);
+    sc.x[t] = (int)((unsigned)sx[t] >> g8);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// One K stage
+// ---------------------------------------------------------------------------------------------
+template <int FMT, int H>
+__device__ __forceinline__ void mfma_one(v16f& acc, v4i w, const typename Fmt<FMT>::xfrag& x, int scw, int scx) {
+  acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(widen(w), widen(x), acc, kFmtE2M1, FMT, 2 * H, scw, 2 * H, scx);
+}
+
+// first copy slot >= K that a stage of format FMT has (slots 4 + x_copies .. 11 are empty)
+template <int FMT>
+constexpr int next_slot(int k) { return (k >= 4 + Fmt<FMT>::x_copies && k < 12) ? 12 : k; }
+
+// 16 MFMAs of one K half.  Between them: the fragment reads of `rd` (for the next half: one after
+// each of the first MFMAs, so that the four waves do not all queue at the LDS at once with their
+// MFMAs stuck behind) and the copy slots [K0, K1) of one stage, one after every second MFMA.
+// LEAN: slots of `lc` into the buffer at byte offset boff; otherwise slots of the run-time plan `gc`.
+template <int FMT, int H, bool LEAN, int M0, int K0, int K1, class Reader>
+__device__ __forceinline__ void mfma_half(v16f (&acc)[4][4], const HalfFrags<FMT>& f, const Scales& sc, const Reader& rd,
+                                          const LeanCopy<FMT>& lc, unsigned boff, const GenericCopy& gc,
+                                          const LaneOffsets& lo, int wave) {
+  if constexpr (M0 < 16) {
+    constexpr int tn = M0 / 4, tm = M0 % 4;
+    mfma_one<FMT, H>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
+    if constexpr (M0 < Reader::kReads) rd.template read<M0>();
+    constexpr int KS = LEAN ? next_slot<FMT>(K0) : K0;
+    if constexpr ((M0 & 1) == 1 && KS < K1) {
+      if constexpr (LEAN) lc.template issue<KS>(boff);
+      else gc.template issue<KS>(lo, wave);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_half<FMT, H, LEAN, M0 + 1, KS + 1, K1>(acc, f, sc, rd, lc, boff, gc, lo, wave);
+    } else {
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_half<FMT, H, LEAN, M0 + 1, K0, K1>(acc, f, sc, rd, lc, boff, gc, lo, wave);
+    }
+  }
+}
+
+// The three stage buffers as byte offsets, rotated once per stage (wave-uniform).
+struct Ring {
+  unsigned cur, nxt, lst;   // buffers of stage q, q+1, q+2
+  __device__ __forceinline__ explicit Ring(int q) {
+    cur = (q % kBuffers) * kStage;
+    nxt = ((q + 1) % kBuffers) * kStage;
+    lst = ((q + 2) % kBuffers) * kStage;
+  }
+  __device__ __forceinline__ void rotate() {
+    const unsigned t = cur;
+    cur = nxt;
+    nxt = lst;
+    lst = t;
+  }
+};
+
+// Stage q of format FMT; FR = format of stage q+1, whose first half is prefetched into `a`
+// (FR == FMT) or `a_next`.  `xp` / `xpn`: token fragment addresses for FMT / FR.
+template <int FMT, int FR, bool LEAN>
+__device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a, HalfFrags<FR>& a_next, Scales& sc,
+                                           LeanCopy<FMT>& lc, GenericCopy& gc, const LaneOffsets& lo, const Plan& plan,
+                                           int q, const Ring& ring, const WeightPtrs& wp, const TokenPtrs<FMT>& xp,
+                                           const TokenPtrs<FR>& xpn, const Ctx& c) {
+  HalfFrags<FMT> b;
+  HalfFrags<FR> nx;
+  v4i sw = {0, 0, 0, 0}, sx = {0, 0, 0, 0};
+  // first half; reads the second half's fragments; the remaining copies of stage q+2 go to the last buffer
+  const FragReader<FMT, 1, false> rd_b{b, sw, sx, wp.w + ring.cur, xp.x + ring.cur, nullptr, nullptr, true};
+  mfma_half<FMT, 0, LEAN, 0, kSplit, kCopySlots>(acc, a, sc, rd_b, lc, ring.lst, gc, lo, c.wave);
+  __builtin_amdgcn_sched_barrier(0);
+  wait_lds_reads();
+#ifdef MG_TICKS
+  const uint64_t tick_b = __builtin_amdgcn_s_memtime();
+#endif
+  if constexpr (LEAN) wait_copies_but_imm<LeanCopy<FMT>::count()>();
+  else wait_copies_but(gc.count());
+  asm volatile("s_barrier" ::: "memory");
+#ifdef MG_TICKS
+  const uint64_t tick_c = __builtin_amdgcn_s_memtime();
+  if (c.lane == 0 && c.wave == 0 && q < 64) {
+    c.ticks[q * 4 + 1] = tick_b;
+    c.ticks[q * 4 + 2] = tick_c;
+  }
+#endif
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (LEAN) lc.advance();
+  else gc = GenericCopy(plan, q + 3, c);
+  // second half; reads the first half and the scales of stage q+1; the first copies of stage q+3
+  // go to the buffer this stage just released
+  const FragReader<FR, 0, true> rd_n{nx, sw, sx, wp.w + ring.nxt, xpn.x + ring.nxt, wp.sw + ring.nxt, wp.sx + ring.nxt,
+                                     LEAN || q + 1 < c.total};
+  mfma_half<FMT, 1, LEAN, 0, 0, kSplit>(acc, b, sc, rd_n, lc, ring.cur, gc, lo, c.wave);
+  __builtin_amdgcn_sched_barrier(0);
+  wait_lds_reads();
+#ifdef MG_TICKS
+  if (c.lane == 0 && c.wave == 0 && q < 64) c.ticks[q * 4 + 3] = __builtin_amdgcn_s_memtime();
+#endif
+  shift_scales(sc, sw, sx, c.lane);
+  if constexpr (FR == FMT) a = nx;
+  else a_next = nx;
+}
+
+// Runs the n >= 1 stages [q0, q0 + n) of one segment whose format is FMT; the next segment has
+// format F1.  On entry `a` holds the first K half of stage q0 and `sc` its scales, `gc` describes
+// stage q0 + 2 (whose first copies are out); on exit `a_next` holds the first half of stage
+// q0 + n when there is one.
+template <int FMT, int F1>
+__device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a, Scales& sc, HalfFrags<F1>& a_next,
+                                            GenericCopy& gc, const LaneOffsets& lo, const Plan& plan, int n, int q0,
+                                            const WeightPtrs& wp, const uint8_t* lds, const Ctx& c) {
+  const TokenPtrs<FMT> xp(lds, c);
+  const TokenPtrs<F1> xpn(lds, c);
+  LeanCopy<FMT> lc;
+  Ring ring(q0);
+  int ql = 0;
+  if (n > 3) {
+    // stages whose stage-after-next-but-one is still in this segment
+    lc.init(plan, q0 + 2, lo, c);
+    for (; ql + 3 < n; ++ql) {
+      HalfFrags<FMT> unused;
+      stage_body<FMT, FMT, true>(acc, a, unused, sc, lc, gc, lo, plan, q0 + ql, ring, wp, xp, xp, c);
+      ring.rotate();
+    }
+    gc = GenericCopy(plan, q0 + ql + 2, c);
+  }
+  for (; ql + 1 < n; ++ql) {
+    HalfFrags<FMT> unused;
+    stage_body<FMT, FMT, false>(acc, a, unused, sc, lc, gc, lo, plan, q0 + ql, ring, wp, xp, xp, c);
+    ring.rotate();
+  }
+  if constexpr (F1 == FMT) {
+    HalfFrags<FMT> unused;
+    stage_body<FMT, FMT, false>(acc, a, unused, sc, lc, gc, lo, plan, q0 + ql, ring, wp, xp, xp, c);
+  } else {
+    stage_body<FMT, F1, false>(acc, a, a_next, sc, lc, gc, lo, plan, q0 + ql, ring, wp, xp, xpn, c);
+  }
+}
+
+#ifdef MG_TICKS
+__device__ uint64_t g_ticks[512];
+#endif
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ d) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  Plan plan;
+  plan.a0 = uni(plan_arg.a0); plan.a1 = uni(plan_arg.a1); plan.a2 = uni(plan_arg.a2);
+  plan.b0 = uni(plan_arg.b0); plan.b1 = uni(plan_arg.b1); plan.b2 = uni(plan_arg.b2);
+  plan.sfa0 = uni(plan_arg.sfa0); plan.sfa1 = uni(plan_arg.sfa1); plan.sfa2 = uni(plan_arg.sfa2);
+  plan.sfb0 = uni(plan_arg.sfb0); plan.sfb1 = uni(plan_arg.sfb1); plan.sfb2 = uni(plan_arg.sfb2);
+  plan.st0 = __builtin_amdgcn_readfirstlane(plan_arg.st0);
+  plan.st1 = __builtin_amdgcn_readfirstlane(plan_arg.st1);
+  plan.st2 = __builtin_amdgcn_readfirstlane(plan_arg.st2);
+  plan.total = __builtin_amdgcn_readfirstlane(plan_arg.total);
+
+  const int tid = threadIdx.x;
+  Ctx c;
+  c.lane = tid & 63;
+  c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  c.wn = c.wave & 1;
+  c.wm = c.wave >> 1;
+  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous band of
+  // feature tiles so that its L2 keeps one slice of the weights.
+  const int wg = blockIdx.x, nwg = gridDim.x;
+  const int tiles_m = nwg / tiles_n;
+  int tile = wg;
+  if ((nwg & 7) == 0) tile = (wg & 7) * (nwg >> 3) + (wg >> 3);
+  c.n0 = (tile / tiles_m) * kT;
+  c.m0 = (tile % tiles_m) * kT;
+  c.total = plan.total;
+  c.lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
+
+  v16f acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
+
+#ifdef MG_TICKS
+  c.ticks = reinterpret_cast<uint64_t*>(lds + kBuffers * kStage);
+  if (tid == 0) c.ticks[0] = __builtin_amdgcn_s_memtime();
+#endif
+  const LaneOffsets lo(plan, c.lane);
+  const WeightPtrs wp(lds, c);
+
+  // prologue: stages 0 and 1 and the first copies of stage 2 in flight; wait for stage 0 only
+  const int n4 = plan.st0, n6 = plan.st1, n8 = plan.st2;
+  GenericCopy gc;
+  {
+    const GenericCopy g0(plan, 0, c);
+    issue_range<0, kCopySlots>(g0, lo, c.wave);
+    const GenericCopy g1(plan, 1, c);
+    issue_range<0, kCopySlots>(g1, lo, c.wave);
+    gc = GenericCopy(plan, 2, c);
+    issue_range<0, kSplit>(gc, lo, c.wave);
+    wait_copies_but(g1.count() + (gc.b.seg < 0 ? 0 : kSplit));
+  }
+  asm volatile("s_barrier" ::: "memory");
+
+  HalfFrags<kFmtE2M1> a4;
+  HalfFrags<kFmtE3M2> a6;
+  HalfFrags<kFmtE4M3> a8, none;
+  Scales sc;
+  {
+    const TokenPtrs<kFmtE2M1> xp(lds, c);
+    v4i sw, sx;
+    const FragReader<kFmtE2M1, 0, true> rd{a4, sw, sx, wp.w, xp.x, wp.sw, wp.sx, true};
+    read_all(rd);
+    wait_lds_reads();
+    shift_scales(sc, sw, sx, c.lane);
+  }
+  run_segment<kFmtE2M1, kFmtE3M2>(acc, a4, sc, a6, gc, lo, plan, n4, 0, wp, lds, c);
+  run_segment<kFmtE3M2, kFmtE4M3>(acc, a6, sc, a8, gc, lo, plan, n6, n4, wp, lds, c);
+  run_segment<kFmtE4M3, kFmtE4M3>(acc, a8, sc, none, gc, lo, plan, n8, n4 + n6, wp, lds, c);
+
+  // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.
+  // Each wave transposes its 128 tokens x 128 features through its own part of the (now idle)
+  // LDS, so that a store instruction writes 4 rows x 256 contiguous bytes instead of 32 rows x 16.
+#ifdef MG_TICKS
+  if (tid == 0 && tile == 77) {
+    for (int i = 0; i < 256; ++i) g_ticks[i] = c.ticks[i];
+    g_ticks[256] = __builtin_amdgcn_s_memtime();
+  }
+#endif
+  constexpr int kPitch = 256 + 16;   // bytes per token row in LDS
+  static_assert(4 * 128 * kPitch <= kBuffers * kStage, "epilogue staging must fit the stage buffers");
+  __syncthreads();                   // every wave is done with the last stage's fragments
+  uint8_t* stage = lds + c.wave * 128 * kPitch;
+  {
+    const int g = c.lane >> 5;
+    uint8_t* wr = stage + (c.lane & 31) * kPitch + 8 * g;
+#pragma unroll
+    for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const v2bf lo2 = {(__bf16)acc[tn][tm][4 * vq + 0], (__bf16)acc[tn][tm][4 * vq + 1]};
+          const v2bf hi2 = {(__bf16)acc[tn][tm][4 * vq + 2], (__bf16)acc[tn][tm][4 * vq + 3]};
+          *reinterpret_cast<v2u*>(wr + tm * 32 * kPitch + tn * 64 + vq * 16) =
+              v2u{__builtin_bit_cast(unsigned, lo2), __builtin_bit_cast(unsigned, hi2)};
+        }
+  }
+  {
+    const int r = c.lane >> 4, cc = c.lane & 15;
+    const uint8_t* rd = stage + r * kPitch + cc * 16;
+    uint16_t* out = d + (size_t)(c.m0 + c.wm * 128 + r) * N + c.n0 + c.wn * 128 + cc * 8;
+#pragma unroll 8
+    for (int i = 0; i < 32; ++i) {
+      const v4u v = *reinterpret_cast<const v4u*>(rd + i * 4 * kPitch);
+      *reinterpret_cast<v4u*>(out + (size_t)i * 4 * N) = v;
+    }
+  }
+}
+
+}  // namespace
+
+#ifdef MG_TICKS
+extern "C" __attribute__((visibility("default"))) int mg_debug_ticks256(unsigned long long* out, int n) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_ticks), (n < 512 ? n : 512) * 8);
+}
+constexpr int kTickBytes = 4096;
+#else
+constexpr int kTickBytes = 0;
+#endif
+
+bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
+  // all three segments present: the pipeline hands the prefetched fragments from one segment's
+  // loop to the next, in the order E2M1 -> E3M2 -> E4M3
+  return M > 0 && N > 0 && M % kT == 0 && N % kT == 0 && KN % 128 == 0 && KS % 128 == 0 && KO % 128 == 0 && KN > 0 &&
+         KS > 0 && KO > 0;
+}
+
+hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
+                                 const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
+                                 const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
+                                 int M, int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mixed_gemm_256_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBuffers * kStage + kTickBytes);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  Plan p;
+  p.a0 = an; p.a1 = as_; p.a2 = ao;
+  p.b0 = bn; p.b1 = bs; p.b2 = bo;
+  p.sfa0 = sfan; p.sfa1 = sfas; p.sfa2 = sfao;
+  p.sfb0 = sfbn; p.sfb1 = sfbs; p.sfb2 = sfbo;
+  p.st0 = KN / 128; p.st1 = KS / 128; p.st2 = KO / 128;
+  p.total = (KN + KS + KO) / 128;
+  const int tiles_n = N / kT, tiles_m = M / kT;
+  hipLaunchKernelGGL(mixed_gemm_256_kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage + kTickBytes, stream, p, tiles_n, N,
+                     static_cast<uint16_t*>(d));
+  return hipGetLastError();
+}
+
+}  // namespace mg

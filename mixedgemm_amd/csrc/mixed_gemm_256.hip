@@ -80,7 +80,10 @@ __device__ __forceinline__ int seg_of(const Plan& p, int q, int& local) {
   return 2;
 }
 
+constexpr int kFmtNone = -1;   // "no stage": copies of a stage past the end of K
+
 template <int FMT> struct Fmt;
+template <> struct Fmt<kFmtNone> { static constexpr int seg = 3, row_bytes = 0, x_copies = 0; typedef v4i xfrag; };
 template <> struct Fmt<kFmtE2M1> { static constexpr int seg = 0, row_bytes = 64, x_copies = 4; typedef v4i xfrag; };
 template <> struct Fmt<kFmtE3M2> { static constexpr int seg = 1, row_bytes = 96, x_copies = 6; typedef v6i xfrag; };
 template <> struct Fmt<kFmtE4M3> { static constexpr int seg = 2, row_bytes = 128, x_copies = 8; typedef v8i xfrag; };
@@ -106,6 +109,8 @@ __device__ __forceinline__ void copy16(const uint8_t* base, unsigned voff, unsig
 // the same with the LDS offset as scalar register + immediate
 template <int OFF>
 __device__ __forceinline__ void copy16i(const uint8_t* base, unsigned voff, unsigned lds_sreg) {
+  base = uni(base);                                         // no-ops when the values are already in scalar registers
+  lds_sreg = __builtin_amdgcn_readfirstlane(lds_sreg);
   asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                : : "v"(voff), "s"(base), "s"(lds_sreg), "n"(OFF) : "memory", "m0", "scc");
 }
@@ -220,24 +225,33 @@ __device__ __forceinline__ void issue_range(const GenericCopy& cp, const LaneOff
 template <int FMT>
 struct LeanCopy {
   static constexpr int NX = Fmt<FMT>::x_copies;
+  // token copies: E2M1 shares the weight offsets (same pitch); E3M2 keeps one offset per third of a
+  // block and E4M3 one, the row step of copy k is added when it is issued (a scalar multiple of lda)
+  static constexpr int NV = FMT == kFmtE2M1 ? 0 : (FMT == kFmtE3M2 ? 3 : 1);
   const uint8_t *w, *x, *s;        // bases of the stage being copied
   unsigned lds_w, lds_x, lds_s;    // LDS offsets of the wave's first weight / token block and scale atom pair in buffer 0
-  unsigned vw[4], vx[NX], vs;
+  unsigned lda;
+  unsigned vw[4], vx[NV > 0 ? NV : 1], vs;
 
-  __device__ __forceinline__ void init(const Plan& plan, int q, const LaneOffsets& lo, const Ctx& c) {
+  __device__ __forceinline__ void init(const Plan& plan, int q, const LaneOffsets&, const Ctx& c) {
+    const LaneOffsets lo(plan, c.lane);   // recomputed here rather than kept in registers across the K loop
     const StageBases b(plan, q, c);
     w = uni(b.w);
     x = uni(b.x);
     s = uni(b.s);
+    lda = __builtin_amdgcn_readfirstlane(b.lda);
     constexpr int sg = Fmt<FMT>::seg;
     const unsigned w_off = sg == 0 ? lo.w0 : (sg == 1 ? lo.w1 : lo.w2);
 #pragma unroll
     for (int k = 0; k < 4; ++k) vw[k] = w_off + k * b.ldb;
-#pragma unroll
-    for (int k = 0; k < NX; ++k) {
-      if constexpr (FMT == kFmtE2M1) vx[k] = vw[k];
-      else if constexpr (FMT == kFmtE3M2) vx[k] = (k % 3 == 0 ? lo.x6a : (k % 3 == 1 ? lo.x6b : lo.x6c)) + (k / 3) * b.lda;
-      else vx[k] = lo.x8 + k * b.lda;
+    if constexpr (FMT == kFmtE3M2) {
+      vx[0] = lo.x6a;
+      vx[1] = lo.x6b;
+      vx[2] = lo.x6c;
+    } else if constexpr (FMT == kFmtE4M3) {
+      vx[0] = lo.x8;
+    } else {
+      vx[0] = 0;
     }
     vs = sg == 0 ? lo.s0 : (sg == 1 ? lo.s1 : lo.s2);
     lds_w = __builtin_amdgcn_readfirstlane(c.lds_base + kWOff + c.wave * 4 * kBlk);
@@ -261,12 +275,23 @@ struct LeanCopy {
       copy16i<K * kBlk>(w, vw[K], lds_w + boff);
     } else if constexpr (K < 4 + NX) {
       constexpr int kx = K - 4;
-      if constexpr (FMT == kFmtE3M2) copy16i<(kx / 3) * kBlk6 + (kx % 3) * 1024>(x, vx[kx], lds_x + boff);
-      else copy16i<kx * kBlk>(x, vx[kx], lds_x + boff);
+      if constexpr (FMT == kFmtE2M1) copy16i<kx * kBlk>(x, vw[kx], lds_x + boff);
+      else if constexpr (FMT == kFmtE3M2)
+        copy16i<(kx / 3) * kBlk6 + (kx % 3) * 1024>(x + (size_t)(kx / 3) * lda, vx[kx % 3], lds_x + boff);
+      else copy16i<kx * kBlk>(x + (size_t)kx * lda, vx[0], lds_x + boff);
     } else if constexpr (K == 12) {
       copy16i<0>(s, vs, lds_s + boff);
     }
   }
+};
+
+template <>
+struct LeanCopy<kFmtNone> {
+  __device__ __forceinline__ void init(const Plan&, int, const LaneOffsets&, const Ctx&) {}
+  __device__ __forceinline__ void advance() {}
+  static constexpr int count() { return 0; }
+  template <int K>
+  __device__ __forceinline__ void issue(unsigned) const {}
 };
 
 // s_waitcnt vmcnt(n) for a run-time, wave-uniform n: the n most recent copies may stay in flight
@@ -413,24 +438,28 @@ constexpr int next_slot(int k) { return (k >= 4 + Fmt<FMT>::x_copies && k < 12) 
 // 16 MFMAs of one K half.  Between them: the fragment reads of `rd` (for the next half: one after
 // each of the first MFMAs, so that the four waves do not all queue at the LDS at once with their
 // MFMAs stuck behind) and the copy slots [K0, K1) of one stage, one after every second MFMA.
-// LEAN: slots of `lc` into the buffer at byte offset boff; otherwise slots of the run-time plan `gc`.
-template <int FMT, int H, bool LEAN, int M0, int K0, int K1, class Reader>
+// LEAN: slots of `lc` (a stage of format CF, skipped when !on) into the buffer at byte offset boff;
+// otherwise slots of the run-time plan `gc`.
+template <int FMT, int H, bool LEAN, int CF, int M0, int K0, int K1, class Reader>
 __device__ __forceinline__ void mfma_half(v16f (&acc)[4][4], const HalfFrags<FMT>& f, const Scales& sc, const Reader& rd,
-                                          const LeanCopy<FMT>& lc, unsigned boff, const GenericCopy& gc,
+                                          const LeanCopy<CF>& lc, bool on, unsigned boff, const GenericCopy& gc,
                                           const LaneOffsets& lo, int wave) {
   if constexpr (M0 < 16) {
     constexpr int tn = M0 / 4, tm = M0 % 4;
     mfma_one<FMT, H>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
     if constexpr (M0 < Reader::kReads) rd.template read<M0>();
-    constexpr int KS = LEAN ? next_slot<FMT>(K0) : K0;
+    constexpr int KS = LEAN ? (CF == kFmtNone ? K1 : next_slot<CF>(K0)) : K0;
     if constexpr ((M0 & 1) == 1 && KS < K1) {
-      if constexpr (LEAN) lc.template issue<KS>(boff);
-      else gc.template issue<KS>(lo, wave);
+      if constexpr (LEAN) {
+        if (on) lc.template issue<KS>(boff);
+      } else {
+        gc.template issue<KS>(lo, wave);
+      }
       __builtin_amdgcn_sched_barrier(0);
-      mfma_half<FMT, H, LEAN, M0 + 1, KS + 1, K1>(acc, f, sc, rd, lc, boff, gc, lo, wave);
+      mfma_half<FMT, H, LEAN, CF, M0 + 1, KS + 1, K1>(acc, f, sc, rd, lc, on, boff, gc, lo, wave);
     } else {
       __builtin_amdgcn_sched_barrier(0);
-      mfma_half<FMT, H, LEAN, M0 + 1, K0, K1>(acc, f, sc, rd, lc, boff, gc, lo, wave);
+      mfma_half<FMT, H, LEAN, CF, M0 + 1, K0, K1>(acc, f, sc, rd, lc, on, boff, gc, lo, wave);
     }
   }
 }
@@ -453,24 +482,34 @@ struct Ring {
 
 // Stage q of format FMT; FR = format of stage q+1, whose first half is prefetched into `a`
 // (FR == FMT) or `a_next`.  `xp` / `xpn`: token fragment addresses for FMT / FR.
-template <int FMT, int FR, bool LEAN>
+// LEAN: the late copy slots (of stage q+2, format CL) come from `lcl` when late_on, the early ones
+// (of stage q+3, format CE) from `lce` when early_on; MID says what happens to `lce` between the
+// halves: 1 = advance by one stage, 2 = set up for stage q+3 (first stage of its segment).
+// !LEAN: both from the run-time plan `gc`.  next_on: there is a stage q+1.
+template <int FMT, int FR, bool LEAN, int CL, int CE, int MID>
 __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a, HalfFrags<FR>& a_next, Scales& sc,
-                                           LeanCopy<FMT>& lc, GenericCopy& gc, const LaneOffsets& lo, const Plan& plan,
-                                           int q, const Ring& ring, const WeightPtrs& wp, const TokenPtrs<FMT>& xp,
+                                           const LeanCopy<CL>& lcl, bool late_on, LeanCopy<CE>& lce, bool early_on,
+                                           GenericCopy& gc, const LaneOffsets& lo, const Plan& plan, int q,
+                                           bool next_on, const Ring& ring, const WeightPtrs& wp, const TokenPtrs<FMT>& xp,
                                            const TokenPtrs<FR>& xpn, const Ctx& c) {
   HalfFrags<FMT> b;
   HalfFrags<FR> nx;
   v4i sw = {0, 0, 0, 0}, sx = {0, 0, 0, 0};
+  wait_lds_reads();   // nothing is outstanding here; tells the compiler so (it cannot see it across the loop edge)
   // first half; reads the second half's fragments; the remaining copies of stage q+2 go to the last buffer
   const FragReader<FMT, 1, false> rd_b{b, sw, sx, wp.w + ring.cur, xp.x + ring.cur, nullptr, nullptr, true};
-  mfma_half<FMT, 0, LEAN, 0, kSplit, kCopySlots>(acc, a, sc, rd_b, lc, ring.lst, gc, lo, c.wave);
+  mfma_half<FMT, 0, LEAN, CL, 0, kSplit, kCopySlots>(acc, a, sc, rd_b, lcl, late_on, ring.lst, gc, lo, c.wave);
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
 #ifdef MG_TICKS
   const uint64_t tick_b = __builtin_amdgcn_s_memtime();
 #endif
-  if constexpr (LEAN) wait_copies_but_imm<LeanCopy<FMT>::count()>();
-  else wait_copies_but(gc.count());
+  if constexpr (LEAN) {
+    if (late_on) wait_copies_but_imm<LeanCopy<CL>::count()>();
+    else wait_copies_but_imm<0>();
+  } else {
+    wait_copies_but(gc.count());
+  }
   asm volatile("s_barrier" ::: "memory");
 #ifdef MG_TICKS
   const uint64_t tick_c = __builtin_amdgcn_s_memtime();
@@ -480,13 +519,17 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
   }
 #endif
   __builtin_amdgcn_sched_barrier(0);
-  if constexpr (LEAN) lc.advance();
-  else gc = GenericCopy(plan, q + 3, c);
+  if constexpr (LEAN) {
+    if constexpr (MID == 1) lce.advance();
+    else if constexpr (MID == 2) lce.init(plan, q + 3, lo, c);
+  } else {
+    gc = GenericCopy(plan, q + 3, c);
+  }
   // second half; reads the first half and the scales of stage q+1; the first copies of stage q+3
   // go to the buffer this stage just released
   const FragReader<FR, 0, true> rd_n{nx, sw, sx, wp.w + ring.nxt, xpn.x + ring.nxt, wp.sw + ring.nxt, wp.sx + ring.nxt,
-                                     LEAN || q + 1 < c.total};
-  mfma_half<FMT, 1, LEAN, 0, 0, kSplit>(acc, b, sc, rd_n, lc, ring.cur, gc, lo, c.wave);
+                                     next_on};
+  mfma_half<FMT, 1, LEAN, CE, 0, 0, kSplit>(acc, b, sc, rd_n, lce, early_on, ring.cur, gc, lo, c.wave);
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
 #ifdef MG_TICKS
@@ -498,38 +541,72 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
 }
 
 // Runs the n >= 1 stages [q0, q0 + n) of one segment whose format is FMT; the next segment has
-// format F1.  On entry `a` holds the first K half of stage q0 and `sc` its scales, `gc` describes
-// stage q0 + 2 (whose first copies are out); on exit `a_next` holds the first half of stage
-// q0 + n when there is one.
-template <int FMT, int F1>
-__device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a, Scales& sc, HalfFrags<F1>& a_next,
-                                            GenericCopy& gc, const LaneOffsets& lo, const Plan& plan, int n, int q0,
-                                            const WeightPtrs& wp, const uint8_t* lds, const Ctx& c) {
+// format F1 (kFmtNone after the last one) and n1 stages; FR1 = F1, or FMT after the last segment.
+// On entry `a` holds the first K half of stage q0 and `sc` its scales; on exit `a_next` holds the
+// first half of stage q0 + n when there is one.
+// REGULAR (every segment but the last has at least 3 stages): `lc` describes the copies of local
+// stage 2 on entry; the last three stages copy the first three of the next segment through
+// `lcn`, which the next segment then continues to use as its `lc`.
+// !REGULAR: `gc` describes stage q0 + 2 (whose first copies are out) on entry and exit; the
+// stages that copy across a segment boundary take the run-time path.
+template <int FMT, int F1, int FR1, bool REGULAR>
+__device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a, Scales& sc, HalfFrags<FR1>& a_next,
+                                            LeanCopy<FMT>& lc, LeanCopy<F1>& lcn, GenericCopy& gc, const LaneOffsets& lo,
+                                            const Plan& plan, int n, int n1, int q0, const WeightPtrs& wp,
+                                            const uint8_t* lds, const Ctx& c) {
   const TokenPtrs<FMT> xp(lds, c);
-  const TokenPtrs<F1> xpn(lds, c);
-  LeanCopy<FMT> lc;
+  const TokenPtrs<FR1> xpn(lds, c);
   Ring ring(q0);
   int ql = 0;
-  if (n > 3) {
-    // stages whose stage-after-next-but-one is still in this segment
-    lc.init(plan, q0 + 2, lo, c);
+  HalfFrags<FMT> unused;
+  if constexpr (REGULAR && F1 != kFmtNone) {
     for (; ql + 3 < n; ++ql) {
-      HalfFrags<FMT> unused;
-      stage_body<FMT, FMT, true>(acc, a, unused, sc, lc, gc, lo, plan, q0 + ql, ring, wp, xp, xp, c);
+      stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, true, lc, true, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+                                              xp, c);
       ring.rotate();
     }
-    gc = GenericCopy(plan, q0 + ql + 2, c);
-  }
-  for (; ql + 1 < n; ++ql) {
-    HalfFrags<FMT> unused;
-    stage_body<FMT, FMT, false>(acc, a, unused, sc, lc, gc, lo, plan, q0 + ql, ring, wp, xp, xp, c);
+    stage_body<FMT, FMT, true, FMT, F1, 2>(acc, a, unused, sc, lc, true, lcn, n1 > 0, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+                                           xp, c);
     ring.rotate();
-  }
-  if constexpr (F1 == FMT) {
-    HalfFrags<FMT> unused;
-    stage_body<FMT, FMT, false>(acc, a, unused, sc, lc, gc, lo, plan, q0 + ql, ring, wp, xp, xp, c);
+    ++ql;
+    stage_body<FMT, FMT, true, F1, F1, 1>(acc, a, unused, sc, lcn, n1 > 0, lcn, n1 > 1, gc, lo, plan, q0 + ql, true, ring, wp,
+                                          xp, xp, c);
+    ring.rotate();
+    ++ql;
+    stage_body<FMT, FR1, true, F1, F1, 1>(acc, a, a_next, sc, lcn, n1 > 1, lcn, n1 > 2, gc, lo, plan, q0 + ql, true, ring, wp,
+                                          xp, xpn, c);
+  } else if constexpr (REGULAR) {
+    // last segment: its own stages only, any n >= 1
+    for (; ql + 1 < n; ++ql) {
+      stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, ql + 2 < n, lc, ql + 3 < n, gc, lo, plan, q0 + ql,
+                                              true, ring, wp, xp, xp, c);
+      ring.rotate();
+    }
+    stage_body<FMT, FMT, true, kFmtNone, kFmtNone, 0>(acc, a, unused, sc, lcn, false, lcn, false, gc, lo, plan, q0 + ql,
+                                                      false, ring, wp, xp, xp, c);
   } else {
-    stage_body<FMT, F1, false>(acc, a, a_next, sc, lc, gc, lo, plan, q0 + ql, ring, wp, xp, xpn, c);
+    if (n > 3) {
+      // stages whose stage-after-next-but-one is still in this segment
+      lc.init(plan, q0 + 2, lo, c);
+      for (; ql + 3 < n; ++ql) {
+        stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, true, lc, true, gc, lo, plan, q0 + ql, true, ring, wp,
+                                                xp, xp, c);
+        ring.rotate();
+      }
+      gc = GenericCopy(plan, q0 + ql + 2, c);
+    }
+    for (; ql + 1 < n; ++ql) {
+      stage_body<FMT, FMT, false, FMT, FMT, 0>(acc, a, unused, sc, lc, true, lc, true, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+                                               xp, c);
+      ring.rotate();
+    }
+    if constexpr (FR1 == FMT) {
+      stage_body<FMT, FMT, false, FMT, FMT, 0>(acc, a, unused, sc, lc, true, lc, true, gc, lo, plan, q0 + ql, false, ring, wp, xp,
+                                               xp, c);
+    } else {
+      stage_body<FMT, FR1, false, FMT, FMT, 0>(acc, a, a_next, sc, lc, true, lc, true, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+                                               xpn, c);
+    }
   }
 }
 
@@ -537,6 +614,7 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a
 __device__ uint64_t g_ticks[512];
 #endif
 
+template <bool REGULAR>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
@@ -608,14 +686,20 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
     wait_lds_reads();
     shift_scales(sc, sw, sx, c.lane);
   }
-  run_segment<kFmtE2M1, kFmtE3M2>(acc, a4, sc, a6, gc, lo, plan, n4, 0, wp, lds, c);
-  run_segment<kFmtE3M2, kFmtE4M3>(acc, a6, sc, a8, gc, lo, plan, n6, n4, wp, lds, c);
-  run_segment<kFmtE4M3, kFmtE4M3>(acc, a8, sc, none, gc, lo, plan, n8, n4 + n6, wp, lds, c);
+  LeanCopy<kFmtE2M1> l4;
+  LeanCopy<kFmtE3M2> l6;
+  LeanCopy<kFmtE4M3> l8;
+  LeanCopy<kFmtNone> l0;
+  if constexpr (REGULAR) l4.init(plan, 2, lo, c);
+  run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
+  run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
+  run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4 + n6, wp, lds, c);
 
   // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.
   // Each wave transposes its 128 tokens x 128 features through its own part of the (now idle)
   // LDS, so that a store instruction writes 4 rows x 256 contiguous bytes instead of 32 rows x 16.
 #ifdef MG_TICKS
+  if (tid == 0 && tile < 250) g_ticks[258 + tile] = __builtin_amdgcn_s_memtime() - c.ticks[0];
   if (tid == 0 && tile == 77) {
     for (int i = 0; i < 256; ++i) g_ticks[i] = c.ticks[i];
     g_ticks[256] = __builtin_amdgcn_s_memtime();
@@ -674,12 +758,15 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
                                  int M, int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mixed_gemm_256_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBuffers * kStage + kTickBytes);
+  // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
+  const bool regular = KN >= 384 && KS >= 384;
+  const void* fn = regular ? reinterpret_cast<const void*>(mixed_gemm_256_kernel<true>)
+                           : reinterpret_cast<const void*>(mixed_gemm_256_kernel<false>);
+  static bool configured[2] = {false, false};
+  if (!configured[regular]) {
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kBuffers * kStage + kTickBytes);
     if (e != hipSuccess) return e;
-    configured = true;
+    configured[regular] = true;
   }
   Plan p;
   p.a0 = an; p.a1 = as_; p.a2 = ao;
@@ -689,8 +776,12 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.st0 = KN / 128; p.st1 = KS / 128; p.st2 = KO / 128;
   p.total = (KN + KS + KO) / 128;
   const int tiles_n = N / kT, tiles_m = M / kT;
-  hipLaunchKernelGGL(mixed_gemm_256_kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage + kTickBytes, stream, p, tiles_n, N,
-                     static_cast<uint16_t*>(d));
+  if (regular)
+    hipLaunchKernelGGL(mixed_gemm_256_kernel<true>, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage + kTickBytes,
+                       stream, p, tiles_n, N, static_cast<uint16_t*>(d));
+  else
+    hipLaunchKernelGGL(mixed_gemm_256_kernel<false>, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage + kTickBytes,
+                       stream, p, tiles_n, N, static_cast<uint16_t*>(d));
   return hipGetLastError();
 }
 

@@ -165,6 +165,8 @@ GEMM_SHAPES = [
     (256, 512, 384, 256, 128), (128, 256, 2560, 1408, 128), (384, 768, 1280, 640, 128),
     # whole 256 x 256 tiles with all three segments: the one-workgroup-per-CU kernel
     (256, 256, 128, 128, 128), (512, 256, 256, 384, 128), (256, 768, 2560, 1408, 128), (512, 512, 640, 256, 256),
+    # the same with at least three 128-wide stages in the first two segments (segment-boundary copies compiled in)
+    (256, 256, 384, 384, 384), (512, 256, 512, 384, 128), (256, 512, 384, 512, 256),
 ]
 
 

@@ -100,18 +100,23 @@ __device__ __forceinline__ void quantize_store(const float (&f)[32], int fmt, ui
   }
 }
 
-// One workgroup handles R consecutive rows; blockDim.x >= K/32 (at most MAXT).
+// A workgroup handles groups of R consecutive rows, group blockIdx.x first and then every
+// gridDim.x-th one; blockDim.x >= K/32 (at most MAXT).  The global loads of the next group are
+// issued before the current group is gathered and quantized, and the LDS tile is double buffered
+// (buf_stride bytes apart; 0 when every workgroup has a single group), so loads, arithmetic and
+// stores of different groups overlap inside the workgroup and one barrier per group suffices.
 template <int R, bool IS_W, int MAXT>
 __global__ void __launch_bounds__(MAXT)
 reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__ idx, int rows, int K, int KN, int KS,
                      int KO, uint8_t* __restrict__ qn, uint8_t* __restrict__ qs, uint8_t* __restrict__ qo,
-                     uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo) {
-  extern __shared__ __align__(16) uint8_t lds[];
+                     uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo, int buf_stride) {
+  extern __shared__ __align__(16) uint8_t lds_all[];
   const int tid = threadIdx.x;
   const int nthr = blockDim.x;
-  const int row0 = blockIdx.x * R;
+  const int ngroups = (rows + R - 1) / R;
 
-  // ---- the lane's 32 reorder indices: requested first, needed only after the barrier
+  // ---- the lane's 32 reorder indices (the same for every row): requested first, needed only
+  //      after the first barrier
   const int b = tid;
   const bool has_block = b < (K >> 5);
   v4u iv[4];
@@ -121,54 +126,7 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
     for (int q = 0; q < 4; ++q) iv[q] = ip[q];
   }
 
-  // ---- stage R rows: all 16-byte loads issued up front (row and chunk clamped instead of
-  //      branched, so nothing waits), R x 8 transpose in registers, 16-byte LDS stores.
-  //      Channel c of row r lands at lds[(c*R + r)*2].
-  const int nchunks = K >> 3;
-  v4u a[4][R];
-#pragma unroll
-  for (int it = 0; it < 4; ++it) {
-    const int c = min(tid + it * nthr, nchunks - 1);
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int row = min(row0 + r, rows - 1);
-      a[it][r] = *reinterpret_cast<const v4u*>(x + (size_t)row * K + (size_t)c * 8);
-    }
-  }
-#pragma unroll
-  for (int it = 0; it < 4; ++it) {
-    const int c = tid + it * nthr;
-    if (c < nchunks) {
-      v4u* dst = reinterpret_cast<v4u*>(lds + (size_t)c * 16 * R);
-      if constexpr (R == 1) {
-        dst[0] = a[it][0];
-      } else if constexpr (R == 2) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          v4u o;
-          o[0] = perm(a[it][1][2 * h], a[it][0][2 * h], 0x05040100u);
-          o[1] = perm(a[it][1][2 * h], a[it][0][2 * h], 0x07060302u);
-          o[2] = perm(a[it][1][2 * h + 1], a[it][0][2 * h + 1], 0x05040100u);
-          o[3] = perm(a[it][1][2 * h + 1], a[it][0][2 * h + 1], 0x07060302u);
-          dst[h] = o;
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          v4u o;
-          o[0] = perm(a[it][1][j], a[it][0][j], 0x05040100u);
-          o[1] = perm(a[it][3][j], a[it][2][j], 0x05040100u);
-          o[2] = perm(a[it][1][j], a[it][0][j], 0x07060302u);
-          o[3] = perm(a[it][3][j], a[it][2][j], 0x07060302u);
-          dst[j] = o;
-        }
-      }
-    }
-  }
-  __syncthreads();
-
-  // ---- one lane per 32-element block
-  if (!has_block) return;
+  // per-lane block constants
   const int nbn = KN >> 5, nbs = KS >> 5;
   const int seg = b < nbn ? 0 : (b < nbn + nbs ? 1 : 2);
   const int j = seg == 0 ? b : (seg == 1 ? b - nbn : b - nbn - nbs);
@@ -180,39 +138,101 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
   uint8_t* qbase = (seg == 0 ? qn : (seg == 1 ? qs : qo)) + j * blk_bytes;
   uint8_t* sfbase = seg == 0 ? sfn : (seg == 1 ? sfs : sfo);
 
-  unsigned g[32][(R + 1) / 2];
-  {
+  // ---- stage R rows: all 16-byte loads issued up front (row and chunk clamped instead of
+  //      branched, so nothing waits), R x 8 transpose in registers, 16-byte LDS stores.
+  //      Channel c of row r lands at lds[(c*R + r)*2].
+  const int nchunks = K >> 3;
+  v4u a[4][R];
+  auto issue_loads = [&](int group) {
+    const int row0 = group * R;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int it = 0; it < 4; ++it) {
+      const int c = min(tid + it * nthr, nchunks - 1);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const unsigned ch = (e & 1) ? (iv[q][e >> 1] >> 16) : (iv[q][e >> 1] & 0xffffu);
-        const int p = q * 8 + e;
-        if constexpr (R == 4) {
-          const v2u d = *reinterpret_cast<const v2u*>(lds + ch * 8);
-          g[p][0] = d[0];
-          g[p][1] = d[1];
+      for (int r = 0; r < R; ++r) {
+        const int row = min(row0 + r, rows - 1);
+        a[it][r] = *reinterpret_cast<const v4u*>(x + (size_t)row * K + (size_t)c * 8);
+      }
+    }
+  };
+
+  int group = blockIdx.x;
+  if (group >= ngroups) return;
+  issue_loads(group);
+  int parity = 0;
+  for (; group < ngroups; group += gridDim.x, parity ^= 1) {
+    uint8_t* lds = lds_all + parity * buf_stride;
+    const int row0 = group * R;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int c = tid + it * nthr;
+      if (c < nchunks) {
+        v4u* dst = reinterpret_cast<v4u*>(lds + (size_t)c * 16 * R);
+        if constexpr (R == 1) {
+          dst[0] = a[it][0];
         } else if constexpr (R == 2) {
-          g[p][0] = *reinterpret_cast<const unsigned*>(lds + ch * 4);
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            v4u o;
+            o[0] = perm(a[it][1][2 * h], a[it][0][2 * h], 0x05040100u);
+            o[1] = perm(a[it][1][2 * h], a[it][0][2 * h], 0x07060302u);
+            o[2] = perm(a[it][1][2 * h + 1], a[it][0][2 * h + 1], 0x05040100u);
+            o[3] = perm(a[it][1][2 * h + 1], a[it][0][2 * h + 1], 0x07060302u);
+            dst[h] = o;
+          }
         } else {
-          g[p][0] = *reinterpret_cast<const uint16_t*>(lds + ch * 2);
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            v4u o;
+            o[0] = perm(a[it][1][jj], a[it][0][jj], 0x05040100u);
+            o[1] = perm(a[it][3][jj], a[it][2][jj], 0x05040100u);
+            o[2] = perm(a[it][1][jj], a[it][0][jj], 0x07060302u);
+            o[3] = perm(a[it][3][jj], a[it][2][jj], 0x07060302u);
+            dst[jj] = o;
+          }
         }
       }
     }
-  }
+    __syncthreads();
+    // the registers are free again: request the next group's rows while this one is processed
+    if (group + (int)gridDim.x < ngroups) issue_loads(group + gridDim.x);
 
+    // ---- one lane per 32-element block
+    if (has_block) {
+      unsigned g[32][(R + 1) / 2];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int row = row0 + r;
-    if (row >= rows) break;
-    float f[32];
+      for (int q = 0; q < 4; ++q) {
 #pragma unroll
-    for (int p = 0; p < 32; ++p) {
-      const unsigned d = g[p][r >> 1];
-      f[p] = __uint_as_float((r & 1) ? (d & 0xffff0000u) : (d << 16));
+        for (int e = 0; e < 8; ++e) {
+          const unsigned ch = (e & 1) ? (iv[q][e >> 1] >> 16) : (iv[q][e >> 1] & 0xffffu);
+          const int p = q * 8 + e;
+          if constexpr (R == 4) {
+            const v2u d = *reinterpret_cast<const v2u*>(lds + ch * 8);
+            g[p][0] = d[0];
+            g[p][1] = d[1];
+          } else if constexpr (R == 2) {
+            g[p][0] = *reinterpret_cast<const unsigned*>(lds + ch * 4);
+          } else {
+            g[p][0] = *reinterpret_cast<const uint16_t*>(lds + ch * 2);
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int row = row0 + r;
+        if (row >= rows) break;
+        float f[32];
+#pragma unroll
+        for (int p = 0; p < 32; ++p) {
+          const unsigned d = g[p][r >> 1];
+          f[p] = __uint_as_float((r & 1) ? (d & 0xffff0000u) : (d << 16));
+        }
+        // per-lane format, code row pitch and byte offset of the block inside its row
+        quantize_store(f, fmt, qbase + (size_t)row * pitch, sfbase + sf_offset(row, j, katoms));
+      }
     }
-    // per-lane format, code row pitch and byte offset of the block inside its row
-    quantize_store(f, fmt, qbase + (size_t)row * pitch, sfbase + sf_offset(row, j, katoms));
+    // with one buffer (buf_stride == 0) there is exactly one group per workgroup; with two, the
+    // barrier of the next iteration separates this gather from the stores two iterations on
   }
 }
 
@@ -225,20 +245,32 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
   if (rows == 0 || K == 0) return hipSuccess;
   const int threads = ((K >> 5) + 63) & ~63;
   const uint16_t* xb = static_cast<const uint16_t*>(x);
-  // R rows interleaved in LDS; keep the tile within 64 KB so several workgroups share a CU
+  // R rows interleaved in LDS.  More row groups than `resident` workgroups: each workgroup
+  // streams several groups through a double-buffered tile.
+  auto launch = [&](auto kernel, int R) {
+    const int tile = K * 2 * R;
+    const int ngroups = ceil_div(rows, R);
+#ifndef MG_QUANT_WGS_PER_CU
+#define MG_QUANT_WGS_PER_CU 4
+#endif
+    int per_cu = (160 * 1024) / (2 * tile);
+    per_cu = per_cu < 1 ? 1 : (per_cu > MG_QUANT_WGS_PER_CU ? MG_QUANT_WGS_PER_CU : per_cu);
+    const int resident = 256 * per_cu;
+    const bool stream_groups = ngroups > resident && 2 * tile <= 160 * 1024;
+    const int grid = stream_groups ? resident : ngroups;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), (size_t)(stream_groups ? 2 * tile : tile), stream, xb, idx, rows, K,
+                       KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream_groups ? tile : 0);
+  };
 #ifndef MG_QUANT_R_SMALLK
-#define MG_QUANT_R_SMALLK 2
+#define MG_QUANT_R_SMALLK 1
 #endif
   if (K <= 8192) {
     constexpr int R = MG_QUANT_R_SMALLK;
-    hipLaunchKernelGGL((reorder_quant_kernel<R, IS_W, 256>), dim3(ceil_div(rows, R)), dim3(threads), (size_t)K * 2 * R,
-                       stream, xb, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+    launch(reorder_quant_kernel<R, IS_W, 256>, R);
   } else if (K <= 16384) {
-    hipLaunchKernelGGL((reorder_quant_kernel<2, IS_W, 512>), dim3(ceil_div(rows, 2)), dim3(threads), (size_t)K * 4, stream,
-                       xb, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+    launch(reorder_quant_kernel<2, IS_W, 512>, 2);
   } else {
-    hipLaunchKernelGGL((reorder_quant_kernel<1, IS_W, 1024>), dim3(rows), dim3(threads), (size_t)K * 2, stream, xb, idx,
-                       rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo);
+    launch(reorder_quant_kernel<1, IS_W, 1024>, 1);
   }
   return hipGetLastError();
 }

@@ -30,6 +30,16 @@ HBM_PEAK_GBS = 8000.0
 P46, P8 = 10100.0, 5000.0
 
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the same
+# counter's reading for `bench.py --calibrate-copy`; None where not measured.  The figures and the
+# commands are in profiles/.
+MEASURED_TRAFFIC = {
+    "gemm_c3": int((154367.6 * 1.9998 + 149632.0 * 1.0) * 1024),   # L2 misses re-read operands ~7x; D written once (+27 %)
+    "quant_c1": int((16453.1 * 1.9998 + 10880.1 * 1.0) * 1024),    # 44.9 MB against 44.2 MB algorithmic
+    "decode_c2": int((18122.4 * 1.9998 + 224.0 * 1.0) * 1024),     # 37.3 MB against 31.4 MB algorithmic
+}
+
+
 def blended_peak(kn, ks, ko):
     return (kn + ks + ko) / ((kn + ks) / P46 + ko / P8)
 
@@ -55,6 +65,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain device copy of known size (256 MiB read + 256 MiB written per launch): "
+                         "the reference point for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -70,6 +83,16 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibrate_copy:
+        src = torch.full((64 << 20,), 3, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "torch copy_ int32", "bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4,
+                          "launches": 5}))
+        return
 
     # ---------------------------------------------------------------- c3
     m, n, k, kn, ks, ko = H.CONFIGS["c3"]
@@ -108,7 +131,7 @@ def main():
     gemm_tflops = flops / (gemm_ms * 1e-3) / 1e12
     roofline = {
         "kernel": "mixed GEMM (c3)", "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": round(peak, 1),
-        "unit": "TFLOP/s", "frac": round(gemm_tflops / peak, 4), "traffic": None,
+        "unit": "TFLOP/s", "frac": round(gemm_tflops / peak, 4), "traffic": MEASURED_TRAFFIC.get("gemm_c3"),
         "avg_kernel_ms": round(gemm_ms, 4), "algorithmic_flops": flops,
     }
 
@@ -121,24 +144,27 @@ def main():
         base = H.make_activations(m1, k1, 1234 + 1).to(dev)
         xs = [base.clone() for _ in range(nsets)]
         outs = [abi.alloc_quant_outputs(m1, kn1, ks1, ko1, abi.MG_OPERAND_A, dev) for _ in range(nsets)]
-        iters = max(args.steps, 40)
+        iters = max(args.steps, 80)
         for i in range(args.warmup + nsets):
             abi.reorder_quantize_x(xs[i % nsets], idx1, kn1, ks1, ko1, out=outs[i % nsets])
         torch.cuda.synchronize()
-        ev1 = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        # one event pair around the whole run of back-to-back launches: a pair per launch would add the
+        # ~3 us event/launch gap to a ~12 us kernel
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         for i in range(iters):
-            ev1[i][0].record()
             abi.reorder_quantize_x(xs[i % nsets], idx1, kn1, ks1, ko1, out=outs[i % nsets])
-            ev1[i][1].record()
+        e1.record()
         torch.cuda.synchronize()
-        q_ms = event_ms(ev1)
+        q_ms = e0.elapsed_time(e1) / iters
         qb = quant_bytes(m1, k1, kn1, ks1, ko1)
         q_gbs = qb / (q_ms * 1e-3) / 1e9
         extra["reorder_quant_c1"] = {
             "workload": "c1 reorder-quantize M=4096 K=4096 (2560/1408/128), random-permutation index, 8 rotating buffer sets",
             "value": round(q_gbs, 1), "unit": "GB/s", "avg_kernel_ms": round(q_ms, 5),
             "roofline": {"bound": "hbm", "achieved": round(q_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": qb},
+                         "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("quant_c1"),
+                         "algorithmic_bytes": qb},
         }
         del xs, outs, base
 
@@ -154,14 +180,14 @@ def main():
             b = wq[i % nsets2]
             abi.matmul(aq2[0], b[0], aq2[1], b[1], aq2[2], b[2], aq2[3], b[3], aq2[4], b[4], aq2[5], b[5], out=d2)
         torch.cuda.synchronize()
-        ev2 = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         for i in range(iters):
             b = wq[i % nsets2]
-            ev2[i][0].record()
             abi.matmul(aq2[0], b[0], aq2[1], b[1], aq2[2], b[2], aq2[3], b[3], aq2[4], b[4], aq2[5], b[5], out=d2)
-            ev2[i][1].record()
+        e1.record()
         torch.cuda.synchronize()
-        g_ms = event_ms(ev2)
+        g_ms = e0.elapsed_time(e1) / iters
         gb = gemm_bytes(m2, n2, kn2, ks2, ko2)
         g_gbs = gb / (g_ms * 1e-3) / 1e9
         extra["decode_gemm_c2"] = {
@@ -169,9 +195,21 @@ def main():
             "value": round(g_gbs, 1), "unit": "GB/s", "avg_kernel_ms": round(g_ms, 5),
             "tflops": round(2.0 * m2 * n2 * k2 / (g_ms * 1e-3) / 1e12, 3),
             "roofline": {"bound": "hbm", "achieved": round(g_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(g_gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": gb},
+                         "frac": round(g_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("decode_c2"),
+                         "algorithmic_bytes": gb},
         }
         del wq
+
+        # ------------------------------------------------------------ what the matrix cores sustain on this box
+        # register-resident scaled-MFMA loop on all CUs: with pseudo-random operand bits the chip hits its
+        # power limit and clocks down, which bounds any GEMM on real data below the nominal peak
+        c_tf, c_ghz = abi.measure_mfma_ceiling(False)
+        r_tf, r_ghz = abi.measure_mfma_ceiling(True)
+        extra["mfma_e2m1_register_loop"] = {
+            "constant_operands": {"tflops": round(c_tf, 1), "shader_ghz": round(c_ghz, 3)},
+            "random_operands": {"tflops": round(r_tf, 1), "shader_ghz": round(r_ghz, 3)},
+            "nominal_peak_tflops": P46,
+        }
 
     # ---------------------------------------------------------------- CPU baseline (oracle, host cores)
     cpu = None

@@ -102,6 +102,13 @@ int mg_device_synchronize(void);
 /* Text for a status code returned by any function above. */
 const char* mg_status_string(int status);
 
+/* Measurement helper with no counterpart in the reference (bench.py reports it next to the
+ * roofline): rate and shader clock at which the whole GPU sustains the E2M1 x E2M1 scaled MFMA
+ * from registers, over `iters` x 16 instructions per wave, with constant (0) or pseudo-random
+ * (1) operand bits.  Allocates and frees its own small buffers, runs on the default stream and
+ * blocks until done.  Returns 0 or a hipError_t. */
+int mg_measure_mfma_ceiling(int random_operands, int iters, double* tflops, double* shader_ghz);
+
 #ifdef __cplusplus
 }
 #endif

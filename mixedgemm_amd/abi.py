@@ -20,6 +20,7 @@ MG_OPERAND_B = 1
 SYMBOLS = (
     "mg_reorder_quantize_x", "mg_reorder_quantize_w", "mg_mixed_gemm", "mg_fused_linear",
     "mg_fused_workspace_bytes", "mg_sf_bytes", "mg_sf_offset", "mg_device_synchronize", "mg_status_string",
+    "mg_measure_mfma_ceiling",
 )
 
 _lib = None
@@ -48,6 +49,8 @@ def lib() -> ctypes.CDLL:
         L.mg_sf_bytes.restype, L.mg_sf_bytes.argtypes = z, [i, i, i]
         L.mg_sf_offset.restype, L.mg_sf_offset.argtypes = z, [i, i, i]
         L.mg_device_synchronize.restype, L.mg_device_synchronize.argtypes = i, []
+        L.mg_measure_mfma_ceiling.restype = i
+        L.mg_measure_mfma_ceiling.argtypes = [i, i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
         L.mg_status_string.restype, L.mg_status_string.argtypes = ctypes.c_char_p, [i]
         _lib = L
     return _lib
@@ -160,6 +163,14 @@ def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, wor
                                    _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
     check(status, "mg_fused_linear")
     return out
+
+
+def measure_mfma_ceiling(random_operands: bool, iters: int = 4000):
+    """(TFLOP/s, shader GHz) of a register-resident E2M1 x E2M1 scaled-MFMA loop on all CUs."""
+    tf, ghz = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    check(lib().mg_measure_mfma_ceiling(int(bool(random_operands)), iters, ctypes.byref(tf), ctypes.byref(ghz)),
+          "mg_measure_mfma_ceiling")
+    return tf.value, ghz.value
 
 
 def device_synchronize() -> None:

@@ -144,9 +144,6 @@ struct LaneOffsets {
 struct Ctx {
   int n0, m0, lane, wave, wn, wm, total;
   unsigned lds_base;   // LDS byte offset of the dynamic shared memory
-#ifdef MG_TICKS
-  uint64_t* ticks;
-#endif
 };
 
 // Wave-uniform bases of the copies of global stage q (any segment).
@@ -501,9 +498,6 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
   mfma_half<FMT, 0, LEAN, CL, 0, kSplit, kCopySlots>(acc, a, sc, rd_b, lcl, late_on, ring.lst, gc, lo, c.wave);
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
-#ifdef MG_TICKS
-  const uint64_t tick_b = __builtin_amdgcn_s_memtime();
-#endif
   if constexpr (LEAN) {
     if (late_on) wait_copies_but_imm<LeanCopy<CL>::count()>();
     else wait_copies_but_imm<0>();
@@ -511,13 +505,6 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
     wait_copies_but(gc.count());
   }
   asm volatile("s_barrier" ::: "memory");
-#ifdef MG_TICKS
-  const uint64_t tick_c = __builtin_amdgcn_s_memtime();
-  if (c.lane == 0 && c.wave == 0 && q < 64) {
-    c.ticks[q * 4 + 1] = tick_b;
-    c.ticks[q * 4 + 2] = tick_c;
-  }
-#endif
   __builtin_amdgcn_sched_barrier(0);
   if constexpr (LEAN) {
     if constexpr (MID == 1) lce.advance();
@@ -532,9 +519,6 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
   mfma_half<FMT, 1, LEAN, CE, 0, 0, kSplit>(acc, b, sc, rd_n, lce, early_on, ring.cur, gc, lo, c.wave);
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
-#ifdef MG_TICKS
-  if (c.lane == 0 && c.wave == 0 && q < 64) c.ticks[q * 4 + 3] = __builtin_amdgcn_s_memtime();
-#endif
   shift_scales(sc, sw, sx, c.lane);
   if constexpr (FR == FMT) a = nx;
   else a_next = nx;
@@ -610,9 +594,6 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a
   }
 }
 
-#ifdef MG_TICKS
-__device__ uint64_t g_ticks[512];
-#endif
 
 template <bool REGULAR>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
@@ -634,14 +615,28 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
   c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   c.wn = c.wave & 1;
   c.wm = c.wave >> 1;
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous band of
-  // feature tiles so that its L2 keeps one slice of the weights.
+  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give each XCD a
+  // contiguous band of feature tiles, and inside the band walk blocks of 8 token tiles, so that
+  // the ~32 tiles an XCD works on at a time share 4 weight tiles and 8 token tiles.
   const int wg = blockIdx.x, nwg = gridDim.x;
   const int tiles_m = nwg / tiles_n;
-  int tile = wg;
-  if ((nwg & 7) == 0) tile = (wg & 7) * (nwg >> 3) + (wg >> 3);
-  c.n0 = (tile / tiles_m) * kT;
-  c.m0 = (tile % tiles_m) * kT;
+  int tile_n = wg / tiles_m, tile_m = wg % tiles_m;
+  if ((nwg & 7) == 0) {
+    const int per_xcd = nwg >> 3;
+    const int j = wg >> 3;                       // position in this XCD's list
+    int tile = (wg & 7) * per_xcd + j;           // feature-major tile index
+    tile_n = tile / tiles_m;
+    tile_m = tile % tiles_m;
+    if (per_xcd % tiles_m == 0 && (tiles_m & 7) == 0) {
+      const int cols = per_xcd / tiles_m;        // feature tiles of the band
+      const int per_block = cols * 8;
+      const int r = j % per_block;
+      tile_n = (wg & 7) * cols + r / 8;
+      tile_m = (j / per_block) * 8 + (r & 7);
+    }
+  }
+  c.n0 = tile_n * kT;
+  c.m0 = tile_m * kT;
   c.total = plan.total;
   c.lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
 
@@ -653,10 +648,6 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
 
-#ifdef MG_TICKS
-  c.ticks = reinterpret_cast<uint64_t*>(lds + kBuffers * kStage);
-  if (tid == 0) c.ticks[0] = __builtin_amdgcn_s_memtime();
-#endif
   const LaneOffsets lo(plan, c.lane);
   const WeightPtrs wp(lds, c);
 
@@ -698,13 +689,6 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
   // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.
   // Each wave transposes its 128 tokens x 128 features through its own part of the (now idle)
   // LDS, so that a store instruction writes 4 rows x 256 contiguous bytes instead of 32 rows x 16.
-#ifdef MG_TICKS
-  if (tid == 0 && tile < 250) g_ticks[258 + tile] = __builtin_amdgcn_s_memtime() - c.ticks[0];
-  if (tid == 0 && tile == 77) {
-    for (int i = 0; i < 256; ++i) g_ticks[i] = c.ticks[i];
-    g_ticks[256] = __builtin_amdgcn_s_memtime();
-  }
-#endif
   constexpr int kPitch = 256 + 16;   // bytes per token row in LDS
   static_assert(4 * 128 * kPitch <= kBuffers * kStage, "epilogue staging must fit the stage buffers");
   __syncthreads();                   // every wave is done with the last stage's fragments
@@ -738,14 +722,6 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
 
 }  // namespace
 
-#ifdef MG_TICKS
-extern "C" __attribute__((visibility("default"))) int mg_debug_ticks256(unsigned long long* out, int n) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_ticks), (n < 512 ? n : 512) * 8);
-}
-constexpr int kTickBytes = 4096;
-#else
-constexpr int kTickBytes = 0;
-#endif
 
 bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
   // all three segments present: the pipeline hands the prefetched fragments from one segment's
@@ -764,7 +740,7 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
                            : reinterpret_cast<const void*>(mixed_gemm_256_kernel<false>);
   static bool configured[2] = {false, false};
   if (!configured[regular]) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kBuffers * kStage + kTickBytes);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kBuffers * kStage);
     if (e != hipSuccess) return e;
     configured[regular] = true;
   }
@@ -777,10 +753,10 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.total = (KN + KS + KO) / 128;
   const int tiles_n = N / kT, tiles_m = M / kT;
   if (regular)
-    hipLaunchKernelGGL(mixed_gemm_256_kernel<true>, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage + kTickBytes,
+    hipLaunchKernelGGL(mixed_gemm_256_kernel<true>, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage,
                        stream, p, tiles_n, N, static_cast<uint16_t*>(d));
   else
-    hipLaunchKernelGGL(mixed_gemm_256_kernel<false>, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage + kTickBytes,
+    hipLaunchKernelGGL(mixed_gemm_256_kernel<false>, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage,
                        stream, p, tiles_n, N, static_cast<uint16_t*>(d));
   return hipGetLastError();
 }

@@ -2,7 +2,7 @@
 // of 4 waves per CU, each wave 128 features x 128 tokens = 4 x 4 tiles of
 // v_mfma_scale_f32_32x32x64_f8f6f4 (256 accumulator registers).  Replaces the three CUTLASS GEMMs
 // of the reference (src/fp4.cu:35, src/fp6.cu:35, src/fp8.cu:35, driver src/gemm.cu:22-47) for
-// M, N multiples of 256 and every K segment a non-empty multiple of 128.
+// M, N multiples of 256 and every K segment at least 128 wide (a multiple of 32).
 //
 // With one wave per SIMD nothing hides a wave's own instruction issue: next to an MFMA (32 cycles
 // in the matrix pipe) a wave gets only a handful of other instructions for free, so the steady
@@ -46,7 +46,8 @@ struct Plan {
   const uint8_t *b0, *b1, *b2;        // weight codes
   const uint8_t *sfa0, *sfa1, *sfa2;  // activation scales
   const uint8_t *sfb0, *sfb1, *sfb2;  // weight scales
-  int st0, st1, st2;                  // stages per segment
+  int st0, st1, st2;                  // whole 128-wide stages per segment
+  int blk0, blk1, blk2;               // 32-element blocks per segment (row pitches and scale atoms; up to 3 more than 4 * st)
   int total;                          // stages over all segments
 };
 
@@ -126,18 +127,18 @@ struct LaneOffsets {
     // quad k of a copy holds tile row j + 16 * (2 * (k % 8) + k / 8): rows 32t + i and 32t + i + 16 of a
     // fragment end up 512 B apart in their block, which the LDS reads conflict-free (64 B apart they collide)
     const unsigned k = lane >> 2, pr = 2 * (k & 7) + (k >> 3), c = lane & 3;
-    w0 = 16 * pr * (p.st0 * 64) + c * 16;
-    w1 = 16 * pr * (p.st1 * 64) + c * 16;
-    w2 = 16 * pr * (p.st2 * 64) + c * 16;
-    x8 = 16 * pr * (p.st2 * 128) + c * 16;
-    const unsigned lda6 = p.st1 * 96, c0 = lane, c1 = 64 + lane, c2 = 128 + lane;
+    w0 = 16 * pr * (p.blk0 * 16) + c * 16;
+    w1 = 16 * pr * (p.blk1 * 16) + c * 16;
+    w2 = 16 * pr * (p.blk2 * 16) + c * 16;
+    x8 = 16 * pr * (p.blk2 * 32) + c * 16;
+    const unsigned lda6 = p.blk1 * 24, c0 = lane, c1 = 64 + lane, c2 = 128 + lane;
     x6a = 8 * (c0 / 6) * lda6 + (c0 % 6) * 16;
     x6b = 8 * (c1 / 6) * lda6 + (c1 % 6) * 16;
     x6c = 8 * (c2 / 6) * lda6 + (c2 % 6) * 16;
     const unsigned hi = lane >> 5, lo = (lane & 31) * 16;
-    s0 = hi * p.st0 * 512 + lo;
-    s1 = hi * p.st1 * 512 + lo;
-    s2 = hi * p.st2 * 512 + lo;
+    s0 = hi * ((p.blk0 + 3) >> 2) * 512 + lo;
+    s1 = hi * ((p.blk1 + 3) >> 2) * 512 + lo;
+    s2 = hi * ((p.blk2 + 3) >> 2) * 512 + lo;
   }
 };
 
@@ -162,10 +163,11 @@ struct StageBases {
     const uint8_t* pb = pick3(sg, plan.b0, plan.b1, plan.b2);
     const uint8_t* psa = pick3(sg, plan.sfa0, plan.sfa1, plan.sfa2);
     const uint8_t* psb = pick3(sg, plan.sfb0, plan.sfb1, plan.sfb2);
-    const unsigned nst = (unsigned)pick3(sg, (uint64_t)plan.st0, (uint64_t)plan.st1, (uint64_t)plan.st2);
+    const unsigned blk = (unsigned)pick3(sg, (uint64_t)plan.blk0, (uint64_t)plan.blk1, (uint64_t)plan.blk2);
+    const unsigned nst = (blk + 3) >> 2;   // scale atoms along K
     const unsigned rb = sg == 0 ? 64 : (sg == 1 ? 96 : 128);
-    ldb = nst * 64;
-    lda = nst * rb;
+    ldb = blk * 16;
+    lda = blk * (rb >> 2);
     w = pb + (size_t)(c.n0 + c.wave * 4) * ldb + (size_t)ql * 64;
     // first token row of the wave: E2M1 4*wave (+kx), E3M2 2*wave (+kx/3), E4M3 8*(wave%2) (+kx) in K half wave/2
     const unsigned xrow = sg == 0 ? c.wave * 4 : (sg == 1 ? c.wave * 2 : (c.wave & 1) * 8);
@@ -595,7 +597,67 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a
 }
 
 
-template <bool REGULAR>
+// The 0..3 blocks of 32 elements a segment has beyond its whole 128-wide stages (e.g. 4928 = 38 * 128
+// + 64): handled after the pipelined stages, straight from global memory, by two more MFMA steps per
+// segment.  Straight-line code: every load is issued (block index clamped into the segment) and
+// absent blocks are turned into zero codes with scale 2^0 afterwards -- branches around code that
+// touches the accumulator make the register allocator spill it.
+template <int FMT>
+__device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                                                 const uint8_t* __restrict__ sfa, const uint8_t* __restrict__ sfb, int blk,
+                                                 const Ctx& c) {
+  const int r = blk & 3, q = blk >> 2;
+  constexpr int XB = Fmt<FMT>::row_bytes / 4;   // token bytes per block
+  const int i = c.lane & 31, g = c.lane >> 5;
+  const int katoms = (blk + 3) >> 2;
+  const unsigned ldb = (unsigned)blk * 16, lda = (unsigned)blk * XB;
+  const v4i z = {0, 0, 0, 0};
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int kb = 2 * h + g;
+    const bool ok = kb < r;
+    const int kbc = min(4 * q + kb, blk - 1);           // a block that exists
+    const int kb1 = min(4 * q + 2 * h + 1, blk - 1);    // E4M3: the second block of the half
+    HalfFrags<FMT> f;
+    Scales sc;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const unsigned n = c.n0 + c.wn * 128 + t * 32 + i, m = c.m0 + c.wm * 128 + t * 32 + i;
+      const v4i wv = *reinterpret_cast<const v4i*>(b + (size_t)n * ldb + (size_t)kbc * 16);
+      const int sw = sfb[sf_offset(n, kbc, katoms)], sx = sfa[sf_offset(m, kbc, katoms)];
+      f.w[t] = ok ? wv : z;
+      sc.w[t] = ok ? sw : 127;
+      sc.x[t] = ok ? sx : 127;
+      const uint8_t* xr = a + (size_t)m * lda;
+      if constexpr (FMT == kFmtE2M1) {
+        const v4i xv = *reinterpret_cast<const v4i*>(xr + (size_t)kbc * 16);
+        f.x[t] = ok ? xv : z;
+      } else if constexpr (FMT == kFmtE3M2) {
+        const v2i* p = reinterpret_cast<const v2i*>(xr + (size_t)kbc * 24);
+        const v2i p0 = p[0], p1 = p[1], p2 = p[2];
+        const v6i xv = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1]};
+        const v6i z6 = {0, 0, 0, 0, 0, 0};
+        f.x[t] = ok ? xv : z6;
+      } else {
+        // K [16g, 16g+16) of the half lies in block 2h, K [32+16g, ...) in block 2h+1
+        const int kb0 = min(4 * q + 2 * h, blk - 1);
+        const v4i pa = *reinterpret_cast<const v4i*>(xr + (size_t)kb0 * 32 + g * 16);
+        const v4i pb = *reinterpret_cast<const v4i*>(xr + (size_t)kb1 * 32 + g * 16);
+        const v4i va = 2 * h < r ? pa : z, vb = 2 * h + 1 < r ? pb : z;
+        f.x[t] = __builtin_shufflevector(va, vb, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm) mfma_one<FMT, 0>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.
+template <bool REGULAR, bool REM>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
@@ -607,6 +669,9 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
   plan.st0 = __builtin_amdgcn_readfirstlane(plan_arg.st0);
   plan.st1 = __builtin_amdgcn_readfirstlane(plan_arg.st1);
   plan.st2 = __builtin_amdgcn_readfirstlane(plan_arg.st2);
+  plan.blk0 = __builtin_amdgcn_readfirstlane(plan_arg.blk0);
+  plan.blk1 = __builtin_amdgcn_readfirstlane(plan_arg.blk1);
+  plan.blk2 = __builtin_amdgcn_readfirstlane(plan_arg.blk2);
   plan.total = __builtin_amdgcn_readfirstlane(plan_arg.total);
 
   const int tid = threadIdx.x;
@@ -686,6 +751,14 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
   run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
   run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4 + n6, wp, lds, c);
 
+  if constexpr (REM) {
+    __builtin_amdgcn_sched_barrier(0);
+    remainder_blocks<kFmtE2M1>(acc, plan.a0, plan.b0, plan.sfa0, plan.sfb0, plan.blk0, c);
+    remainder_blocks<kFmtE3M2>(acc, plan.a1, plan.b1, plan.sfa1, plan.sfb1, plan.blk1, c);
+    remainder_blocks<kFmtE4M3>(acc, plan.a2, plan.b2, plan.sfa2, plan.sfb2, plan.blk2, c);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
   // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.
   // Each wave transposes its 128 tokens x 128 features through its own part of the (now idle)
   // LDS, so that a store instruction writes 4 rows x 256 contiguous bytes instead of 32 rows x 16.
@@ -724,10 +797,10 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
 
 
 bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
-  // all three segments present: the pipeline hands the prefetched fragments from one segment's
-  // loop to the next, in the order E2M1 -> E3M2 -> E4M3
-  return M > 0 && N > 0 && M % kT == 0 && N % kT == 0 && KN % 128 == 0 && KS % 128 == 0 && KO % 128 == 0 && KN > 0 &&
-         KS > 0 && KO > 0;
+  // all three segments with at least one whole 128-wide stage: the pipeline hands the prefetched
+  // fragments from one segment's loop to the next, in the order E2M1 -> E3M2 -> E4M3
+  return M > 0 && N > 0 && M % kT == 0 && N % kT == 0 && KN % 32 == 0 && KS % 32 == 0 && KO % 32 == 0 && KN >= 128 &&
+         KS >= 128 && KO >= 128;
 }
 
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
@@ -735,14 +808,18 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
                                  int M, int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
   // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
-  const bool regular = KN >= 384 && KS >= 384;
-  const void* fn = regular ? reinterpret_cast<const void*>(mixed_gemm_256_kernel<true>)
-                           : reinterpret_cast<const void*>(mixed_gemm_256_kernel<false>);
-  static bool configured[2] = {false, false};
-  if (!configured[regular]) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kBuffers * kStage);
+  const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
+  const bool rem = (KN | KS | KO) % 128 != 0;
+  typedef void (*kernel_t)(Plan, int, int, uint16_t*);
+  const kernel_t kernels[2][2] = {{mixed_gemm_256_kernel<false, false>, mixed_gemm_256_kernel<false, true>},
+                                  {mixed_gemm_256_kernel<true, false>, mixed_gemm_256_kernel<true, true>}};
+  const kernel_t kernel = kernels[regular][rem];
+  static bool configured[2][2] = {{false, false}, {false, false}};
+  if (!configured[regular][rem]) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       kBuffers * kStage);
     if (e != hipSuccess) return e;
-    configured[regular] = true;
+    configured[regular][rem] = true;
   }
   Plan p;
   p.a0 = an; p.a1 = as_; p.a2 = ao;
@@ -750,14 +827,11 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.sfa0 = sfan; p.sfa1 = sfas; p.sfa2 = sfao;
   p.sfb0 = sfbn; p.sfb1 = sfbs; p.sfb2 = sfbo;
   p.st0 = KN / 128; p.st1 = KS / 128; p.st2 = KO / 128;
-  p.total = (KN + KS + KO) / 128;
+  p.blk0 = KN / 32; p.blk1 = KS / 32; p.blk2 = KO / 32;
+  p.total = p.st0 + p.st1 + p.st2;
   const int tiles_n = N / kT, tiles_m = M / kT;
-  if (regular)
-    hipLaunchKernelGGL(mixed_gemm_256_kernel<true>, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage,
-                       stream, p, tiles_n, N, static_cast<uint16_t*>(d));
-  else
-    hipLaunchKernelGGL(mixed_gemm_256_kernel<false>, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage,
-                       stream, p, tiles_n, N, static_cast<uint16_t*>(d));
+  hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage, stream, p, tiles_n, N,
+                     static_cast<uint16_t*>(d));
   return hipGetLastError();
 }
 

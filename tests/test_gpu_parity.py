@@ -167,6 +167,8 @@ GEMM_SHAPES = [
     (256, 256, 128, 128, 128), (512, 256, 256, 384, 128), (256, 768, 2560, 1408, 128), (512, 512, 640, 256, 256),
     # the same with at least three 128-wide stages in the first two segments (segment-boundary copies compiled in)
     (256, 256, 384, 384, 384), (512, 256, 512, 384, 128), (256, 512, 384, 512, 256),
+    # segments that end 32, 64 or 96 elements past their last whole 128-wide stage
+    (256, 256, 448, 416, 224), (256, 512, 2240, 1248, 448), (512, 256, 160, 480, 352),
 ]
 
 

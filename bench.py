@@ -166,6 +166,26 @@ def main():
                          "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("quant_c1"),
                          "algorithmic_bytes": qb},
         }
+        # ------------------------------------------------------------ calibration: column absmax + sort (reads X once)
+        wsp = torch.empty(int(abi.lib().mg_calibrate_workspace_bytes(k1)), dtype=torch.uint8, device=dev)
+        idx_out = torch.empty(k1, dtype=torch.int16, device=dev)
+        for i in range(args.warmup):
+            abi.calibrate_reorder_index(xs[i % nsets], out=idx_out, workspace=wsp)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(iters):
+            abi.calibrate_reorder_index(xs[i % nsets], out=idx_out, workspace=wsp)
+        e1.record()
+        torch.cuda.synchronize()
+        c_ms = e0.elapsed_time(e1) / iters
+        cb = m1 * k1 * 2 + k1 * 2
+        extra["calibrate_index_c1"] = {
+            "workload": "reorder index of the c1 activations: per-channel absmax over M=4096 rows + sort of K=4096 channels",
+            "value": round(cb / (c_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "avg_ms": round(c_ms, 5),
+            "roofline": {"bound": "hbm", "achieved": round(cb / (c_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(cb / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": cb},
+        }
         del xs, outs, base
 
         # ------------------------------------------------------------ c2: decode GEMM, HBM-bound

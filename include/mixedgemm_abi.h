@@ -95,6 +95,14 @@ size_t mg_sf_bytes(int rows, int kseg, int operand);
  * scale buffer (include/reorder.cuh:119-124; src/reorder.cu:182-185). */
 size_t mg_sf_offset(int row, int kb, int kseg);
 
+/* Calibration step that produces the reorder index (the commented lines main.py:31-33 of the
+ * reference: per-channel max |x| over the rows of a bf16 sample X[M,K], channels sorted by it in
+ * ascending order, as int16).  Ties are ordered by channel number.  K a multiple of 32, <= 32736.
+ * `workspace`: mg_calibrate_workspace_bytes(K) bytes of device memory, 16-byte aligned. */
+int mg_calibrate_reorder_index(const void* x_bf16, int M, int K, int16_t* idx,
+                               void* workspace, size_t workspace_bytes, void* stream);
+size_t mg_calibrate_workspace_bytes(int K);
+
 /* Blocks the host until all work on the current device has finished
  * (src/bindings.cpp:59,178,297 do this after every operator). */
 int mg_device_synchronize(void);

@@ -20,7 +20,7 @@ MG_OPERAND_B = 1
 SYMBOLS = (
     "mg_reorder_quantize_x", "mg_reorder_quantize_w", "mg_mixed_gemm", "mg_fused_linear",
     "mg_fused_workspace_bytes", "mg_sf_bytes", "mg_sf_offset", "mg_device_synchronize", "mg_status_string",
-    "mg_measure_mfma_ceiling",
+    "mg_measure_mfma_ceiling", "mg_calibrate_reorder_index", "mg_calibrate_workspace_bytes",
 )
 
 _lib = None
@@ -49,6 +49,8 @@ def lib() -> ctypes.CDLL:
         L.mg_sf_bytes.restype, L.mg_sf_bytes.argtypes = z, [i, i, i]
         L.mg_sf_offset.restype, L.mg_sf_offset.argtypes = z, [i, i, i]
         L.mg_device_synchronize.restype, L.mg_device_synchronize.argtypes = i, []
+        L.mg_calibrate_reorder_index.restype, L.mg_calibrate_reorder_index.argtypes = i, [p, i, i, p, p, z, p]
+        L.mg_calibrate_workspace_bytes.restype, L.mg_calibrate_workspace_bytes.argtypes = z, [i]
         L.mg_measure_mfma_ceiling.restype = i
         L.mg_measure_mfma_ceiling.argtypes = [i, i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
         L.mg_status_string.restype, L.mg_status_string.argtypes = ctypes.c_char_p, [i]
@@ -162,6 +164,22 @@ def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, wor
                                    _ptr(sfbn), _ptr(sfbs), _ptr(sfbo), m, n, kn, ks, ko,
                                    _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
     check(status, "mg_fused_linear")
+    return out
+
+
+def calibrate_reorder_index(x, out=None, workspace=None):
+    """Reorder index of a bf16 activation sample x[M, K]: channels by ascending max |x| over the
+    rows, ties by channel number, int16 (main.py:31-33 of the reference, there as torch calls)."""
+    _require(x, torch.bfloat16, "x")
+    assert x.dim() == 2
+    m, k = x.shape
+    need = int(lib().mg_calibrate_workspace_bytes(k))
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = torch.empty(k, dtype=torch.int16, device=x.device)
+    check(lib().mg_calibrate_reorder_index(_ptr(x), m, k, _ptr(out), _ptr(workspace), workspace.numel(),
+                                           _stream(x)), "mg_calibrate_reorder_index")
     return out
 
 

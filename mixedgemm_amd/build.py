@@ -22,7 +22,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libmixedgemm_hip.so")
 EXT_DIR = os.path.join(ROOT, "build")
 EXT_PATH = os.path.join(EXT_DIR, "mixedgemm.so")
 
-HIP_SOURCES = ["abi.hip", "reorder_quant.hip", "mixed_gemm.hip", "mixed_gemm_256.hip", "ceiling.hip"]
+HIP_SOURCES = ["abi.hip", "reorder_quant.hip", "mixed_gemm.hip", "mixed_gemm_256.hip", "calibrate.hip", "ceiling.hip"]
 HIP_HEADERS = ["mg_common.h", os.path.join(ROOT, "include", "mixedgemm_abi.h")]
 
 HIPCC_FLAGS = [

@@ -13,6 +13,8 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
                              int N, int KN, int KS, int KO, void* d, hipStream_t stream);
+size_t calibrate_workspace_bytes(int K);
+hipError_t launch_calibrate(const void* x, int rows, int K, int16_t* idx, void* workspace, hipStream_t stream);
 }  // namespace mg
 
 namespace {
@@ -109,6 +111,17 @@ int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, c
   uint8_t* sfo = p;
   if (int s = mg_reorder_quantize_x(x_bf16, idx, M, KN + KS + KO, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream)) return s;
   return mg_mixed_gemm(qn, bn, qs, bs, qo, bo, sfn, sfbn, sfs, sfbs, sfo, sfbo, M, N, KN, KS, KO, d_bf16, stream);
+}
+
+size_t mg_calibrate_workspace_bytes(int K) { return K > 0 ? mg::calibrate_workspace_bytes(K) : 0; }
+
+int mg_calibrate_reorder_index(const void* x_bf16, int M, int K, int16_t* idx, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  if (M <= 0 || K <= 0 || (K & 31)) return MG_ERR_BAD_SHAPE;
+  if (K > 32736) return MG_ERR_UNSUPPORTED;
+  if (!x_bf16 || !aligned16(x_bf16) || !idx || !workspace || !aligned16(workspace)) return MG_ERR_BAD_POINTER;
+  if (workspace_bytes < mg::calibrate_workspace_bytes(K)) return MG_ERR_BAD_SHAPE;
+  return (int)mg::launch_calibrate(x_bf16, M, K, idx, workspace, static_cast<hipStream_t>(stream));
 }
 
 int mg_device_synchronize(void) { return (int)hipDeviceSynchronize(); }

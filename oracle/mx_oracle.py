@@ -336,3 +336,13 @@ def fake_quant_linear(x, w, idx, kn, ks, ko):
     qx = reorder_quantize_x(x, idx, kn, ks, ko)
     qw = reorder_quantize_w(w, idx, kn, ks, ko)
     return bf16_rne(mixed_matmul(qx, qw))
+
+
+def calibrate_reorder_index(x_bits):
+    """Reorder index of a bf16 sample given as uint16 bit patterns [M, K]: channels by ascending
+    per-channel max |x|, ties by channel number, int16 (main.py:31-33 of the reference:
+    torch.max(torch.abs(X), dim=0).values -> torch.sort ascending -> int16; torch leaves the order
+    of ties open, here it is fixed).  For finite values the bf16 bit pattern with the sign cleared
+    orders like |x|, so no float conversion is needed."""
+    mag = (np.asarray(x_bits, dtype=np.uint16) & 0x7FFF).max(axis=0).astype(np.uint32)
+    return np.argsort(mag, kind="stable").astype(np.int16)

@@ -286,3 +286,19 @@ def test_extension_module_runs_the_reference_call_sequence(abi):
     _check_gemm(C, qx, qw, "extension")
     with pytest.raises(RuntimeError):
         mixedgemm.reorder_quantize_x(xd, idd.to(torch.int32), kn, ks, ko, m, n)
+
+
+@pytest.mark.parametrize("m,k", [(1, 32), (7, 96), (64, 4096), (129, 2080), (300, 14336), (4096, 4096), (33, 32736)])
+def test_calibrate_reorder_index_matches_oracle(abi, m, k):
+    """Per-channel absmax + stable ascending sort: identical index to the oracle, including the
+    order of ties (coarse values make many) and channels that are entirely zero."""
+    _say("calibrate", m, k)
+    g = torch.Generator().manual_seed(m * 131 + k)
+    if k <= 4096:
+        x = (torch.randint(-6, 7, (m, k), generator=g).float() * 0.25).bfloat16()    # many ties
+        x[:, ::17] = 0
+    else:
+        x = H.make_activations(m, k, m + k)
+    idx = abi.calibrate_reorder_index(x.cuda())
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(idx.cpu().numpy(), mo.calibrate_reorder_index(H.bf16_bits(x)))

@@ -326,3 +326,36 @@ def test_chain_mode_rounds_three_times():
     chained = mo.mixed_matmul(qx, qw, chain_bf16=True)
     np.testing.assert_array_equal(chained, mo.bf16_rne(chained))
     np.testing.assert_allclose(chained, full, rtol=3 * 2.0 ** -8, atol=1e-3)
+
+
+# ---------------------------------------------------------------- calibration (reorder index)
+def test_calibrate_index_matches_torch_sort_of_absmax():
+    """The reference's recipe run literally on the CPU (torch.max(torch.abs(X), dim=0) ->
+    torch.sort ascending -> int16, main.py:31-33), on data without ties where its result is
+    unique, and with stable=True on data full of ties."""
+    from tests import helpers as H
+    g = torch.Generator().manual_seed(11)
+    # 256 distinct bf16 magnitudes (consecutive bit patterns from 1.0 up), one per channel, as the
+    # channel maxima; the other rows stay below them
+    peak = (torch.arange(256, dtype=torch.int32) + 0x3F80).to(torch.int16).view(torch.bfloat16)[torch.randperm(256, generator=g)]
+    x = (torch.rand(37, 256, generator=g) * 0.9 * peak.float()).bfloat16()
+    x[11] = peak * (torch.randint(0, 2, (256,), generator=g) * 2 - 1).bfloat16()
+    absmax = torch.max(torch.abs(x.float()), dim=0).values
+    assert absmax.unique().numel() == absmax.numel()
+    ref = torch.sort(absmax, descending=False).indices.to(torch.int16).numpy()
+    np.testing.assert_array_equal(mo.calibrate_reorder_index(H.bf16_bits(x)), ref)
+    # ties: few distinct magnitudes, negative zeros, a zero channel
+    t = (torch.randint(-3, 4, (19, 128), generator=g).float() * 0.5).bfloat16()
+    t[:, 5] = 0.0
+    t[3, 7] = -0.0
+    ref = torch.sort(torch.max(torch.abs(t.float()), dim=0).values, descending=False, stable=True).indices.to(torch.int16).numpy()
+    np.testing.assert_array_equal(mo.calibrate_reorder_index(H.bf16_bits(t)), ref)
+
+
+def test_calibrate_index_is_a_permutation_sorted_by_absmax():
+    from tests import helpers as H
+    x = H.make_activations(64, 4096, 5)
+    idx = mo.calibrate_reorder_index(H.bf16_bits(x)).astype(np.int64)
+    assert sorted(idx.tolist()) == list(range(4096))
+    am = x.float().abs().max(dim=0).values.numpy()
+    assert np.all(np.diff(am[idx]) >= 0)

@@ -1,0 +1,94 @@
+"""GPU tests of the caller layer: packed-weight file, registered torch operators on a side
+stream, and the linear layer, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mx_oracle as mo
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def linear():
+    from mixedgemm_amd import abi, linear as l
+    abi.lib()
+    return l
+
+
+def _oracle_linear(x, w, idx, split):
+    qx = mo.reorder_quantize_x(H.bf16_f32(x), idx.numpy(), *split)
+    qw = mo.reorder_quantize_w(H.bf16_f32(w), idx.numpy(), *split)
+    ref = mo.mixed_matmul(qx, qw)
+    slack = (np.abs(mo.dequantize_x(qx)).astype(np.float64) @ np.abs(mo.dequantize_w(qw)).astype(np.float64).T) * 2.0 ** -20
+    return ref, slack
+
+
+def _close(d, ref, slack):
+    err = np.abs(d.float().cpu().numpy() - mo.bf16_rne(ref))
+    assert np.all(err <= H.bf16_ulp(ref) + slack), f"max err {err.max()}"
+
+
+@pytest.mark.parametrize("m,n,k", [(24, 64, 4096), (3, 32, 3584), (256, 256, 5120)])
+def test_linear_layer_matches_oracle(linear, m, n, k):
+    print("linear layer", m, n, k, flush=True)
+    split = linear.default_split(k)
+    x = H.make_activations(m, k, 900 + m)
+    w = H.make_weights(n, k, 901 + m)
+    layer = linear.MixedLinear.from_float(w.to(DEV), calibration_x=x.to(DEV))
+    idx = H.absmax_sort_index(x)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(layer.reorder_index.cpu().numpy(), idx.numpy())
+    y = layer(x.to(DEV).reshape(1, m, k))
+    torch.cuda.synchronize()
+    assert y.shape == (1, m, n)
+    ref, slack = _oracle_linear(x, w, idx, split)
+    _close(y[0], ref, slack)
+
+
+def test_pack_file_round_trip_through_the_gpu(linear, tmp_path):
+    m, n, k = 16, 48, 4096
+    split = linear.default_split(k)
+    x = H.make_activations(m, k, 77)
+    w = H.make_weights(n, k, 78)
+    idx = H.absmax_sort_index(x)
+    pw = linear.PackedWeights.from_float(w.to(DEV), idx.to(DEV), split)
+    torch.cuda.synchronize()
+    path = str(tmp_path / "layer.mgw")
+    pw.save(path)
+    back = linear.PackedWeights.load(path, device=DEV)
+    for a, b in zip((*pw.tensors(), pw.reorder_index), (*back.tensors(), back.reorder_index)):
+        assert torch.equal(a, b)
+    y0 = linear.MixedLinear(pw)(x.to(DEV))
+    y1 = linear.MixedLinear(back)(x.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(y0, y1)
+    ref, slack = _oracle_linear(x, w, idx, split)
+    _close(y1, ref, slack)
+
+
+def test_operators_run_on_the_current_stream_without_synchronizing(linear):
+    """The three reference calls as registered operators on a side stream: results are complete
+    after waiting for that stream only, and equal those of the default stream."""
+    m, n, k = 40, 64, 4096
+    kn, ks, ko = linear.default_split(k)
+    x = H.make_activations(m, k, 5).to(DEV)
+    w = H.make_weights(n, k, 6).to(DEV)
+    idx = torch.ops.mixedgemm_amd.calibrate_reorder_index(x)
+    ops = torch.ops.mixedgemm_amd
+    a = ops.reorder_quantize_x(x, idx, kn, ks, ko)
+    b = ops.reorder_quantize_w(w, idx, kn, ks, ko)
+    d0 = ops.matmul(a[0], b[0], a[1], b[1], a[2], b[2], a[3], b[3], a[4], b[4], a[5], b[5])
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        a1 = ops.reorder_quantize_x(x, idx, kn, ks, ko)
+        d1 = ops.matmul(a1[0], b[0], a1[1], b[1], a1[2], b[2], a1[3], b[3], a1[4], b[4], a1[5], b[5])
+        d2 = ops.fused_linear(x, idx, *b, kn, ks, ko)
+    side.synchronize()
+    assert torch.equal(d0, d1) and torch.equal(d0, d2)
+    for t0, t1 in zip(a[:3], a1[:3]):
+        assert torch.equal(t0, t1)

@@ -302,3 +302,36 @@ def test_calibrate_reorder_index_matches_oracle(abi, m, k):
     idx = abi.calibrate_reorder_index(x.cuda())
     torch.cuda.synchronize()
     np.testing.assert_array_equal(idx.cpu().numpy(), mo.calibrate_reorder_index(H.bf16_bits(x)))
+
+
+# ------------------------------------------------------------------ committed golden vectors
+import glob as _glob
+import os as _os
+
+GOLDEN = sorted(_glob.glob(_os.path.join(_os.path.dirname(__file__), "golden", "path_*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[_os.path.basename(p) for p in GOLDEN])
+def test_whole_path_matches_golden_vectors(abi, path):
+    """Calibrate -> quantize both operands -> GEMM, on the inputs of a committed fixture."""
+    _say("golden", _os.path.basename(path))
+    g = np.load(path)
+    kn, ks, ko = (int(v) for v in g["split"])
+    x = torch.from_numpy(g["x_bits"].view(np.int16)).view(torch.bfloat16).to(DEV)
+    w = torch.from_numpy(g["w_bits"].view(np.int16)).view(torch.bfloat16).to(DEV)
+    idx = abi.calibrate_reorder_index(x)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(idx.cpu().numpy(), g["idx"])
+    aq = abi.reorder_quantize_x(x, idx, kn, ks, ko)
+    bq = abi.reorder_quantize_w(w, idx, kn, ks, ko)
+    d = abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5])
+    torch.cuda.synchronize()
+    for tag, q, rows in (("x", aq, x.shape[0]), ("w", bq, w.shape[0])):
+        for t, c in zip(q[:3], ("qn", "qs", "qo")):
+            np.testing.assert_array_equal(t.cpu().numpy(), g[f"{tag}_{c}"], err_msg=f"{tag} {c}")
+        for t, s, kseg in zip(q[3:], ("sfn", "sfs", "sfo"), (kn, ks, ko)):
+            np.testing.assert_array_equal(H.gather_logical_scales(t, rows, kseg), g[f"{tag}_{s}"], err_msg=f"{tag} {s}")
+    ref = g["d_f32"]
+    err = np.abs(d.float().cpu().numpy() - mo.bf16_rne(ref))
+    # 1 bf16 ulp for the final rounding + 2^-20 of sum |a||b| for the order of the fp32 accumulation
+    assert np.all(err <= H.bf16_ulp(ref) + g["d_abs_f32"] * 2.0 ** -20), f"max err {err.max()}"

@@ -220,6 +220,48 @@ def main():
         }
         del wq
 
+        # ------------------------------------------------------------ the other layer shapes of the reference's K list
+        # fused step (activation reorder-quantize + mixed GEMM) per shape; weights quantized outside the timing
+        from mixedgemm_amd import linear as caller
+        matrix = []
+        shapes = [("c0", 128, 4096, 4096), ("c4", 2048, 4096, 14336), ("", 4096, 13824, 5120), ("", 4096, 5120, 13824),
+                  ("", 4096, 18944, 3584), ("", 4096, 3584, 18944), ("", 4096, 4096, 12288)]
+        for tag, mm, nn, kk in shapes:
+            knm, ksm, kom = caller.default_split(kk)
+            xm = H.make_activations(mm, kk, 1234 + 4, student_t=(tag == "c4")).to(dev)
+            idm = abi.calibrate_reorder_index(xm)
+            wqm = abi.reorder_quantize_w(H.make_weights(nn, kk, 2234 + 4).to(dev), idm, knm, ksm, kom)
+            aqm = abi.alloc_quant_outputs(mm, knm, ksm, kom, abi.MG_OPERAND_A, dev)
+            dm = torch.empty((mm, nn), dtype=torch.bfloat16, device=dev)
+
+            def quant():
+                abi.reorder_quantize_x(xm, idm, knm, ksm, kom, out=aqm)
+
+            def gemm():
+                abi.matmul(aqm[0], wqm[0], aqm[1], wqm[1], aqm[2], wqm[2], aqm[3], wqm[3], aqm[4], wqm[4], aqm[5], wqm[5], out=dm)
+
+            times = []
+            for fn in (quant, gemm):
+                for _ in range(5):
+                    fn()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(20):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                times.append(e0.elapsed_time(e1) / 20)
+            flops = 2.0 * mm * nn * kk
+            matrix.append({"config": tag, "M": mm, "N": nn, "K": kk, "split": [knm, ksm, kom],
+                           "quant_ms": round(times[0], 5), "gemm_ms": round(times[1], 5),
+                           "gemm_tflops": round(flops / (times[1] * 1e-3) / 1e12, 1),
+                           "fused_tflops": round(flops / ((times[0] + times[1]) * 1e-3) / 1e12, 1),
+                           "quant_gbs": round(quant_bytes(mm, kk, knm, ksm, kom) / (times[0] * 1e-3) / 1e9, 1)})
+            del xm, wqm, aqm, dm
+        extra["shape_matrix"] = {"note": "back-to-back launches on one buffer set (operands may sit in the 256 MB "
+                                         "Infinity Cache); 5 warm-up + 20 timed launches per kernel", "rows": matrix}
+
         # ------------------------------------------------------------ what the matrix cores sustain on this box
         # register-resident scaled-MFMA loop on all CUs: with pseudo-random operand bits the chip hits its
         # power limit and clocks down, which bounds any GEMM on real data below the nominal peak

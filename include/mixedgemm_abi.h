@@ -74,6 +74,22 @@ int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, cons
                   int M, int N, int KN, int KS, int KO, void* d_bf16, void* stream);
 
 /*
+ * The same GEMM for a caller whose activation buffers have room for more token rows than M:
+ * an, as_, ao are readable for a_rows >= M rows and sfan, sfas, sfao for
+ * mg_sf_bytes(a_rows, kseg, MG_OPERAND_A) bytes (what lies past row M is never used for a result).
+ * With a_rows >= mg_padded_rows(M) a token count that is not a multiple of 256 runs on the
+ * whole-tile kernel like any other; with a_rows == M this is mg_mixed_gemm.  The reference has
+ * no counterpart: its CUTLASS GEMMs (src/fp4.cu:164-182) predicate partial tiles themselves.
+ */
+int mg_mixed_gemm_rows(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
+                       const uint8_t* ao, const uint8_t* bo,
+                       const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
+                       const uint8_t* sfao, const uint8_t* sfbo,
+                       int M, int a_rows, int N, int KN, int KS, int KO, void* d_bf16, void* stream);
+/* M rounded up to whole 256-token tiles. */
+int mg_padded_rows(int M);
+
+/*
  * Activation reorder-quantize followed by the mixed GEMM on the same stream
  * (the sequence src/bindings.cpp:69-186 then :9-67 performs with a device-wide
  * synchronize in between; bench_reorder_gemm.cu:163-167 times the same pair).

@@ -18,7 +18,8 @@ MG_OPERAND_A = 0
 MG_OPERAND_B = 1
 
 SYMBOLS = (
-    "mg_reorder_quantize_x", "mg_reorder_quantize_w", "mg_mixed_gemm", "mg_fused_linear",
+    "mg_reorder_quantize_x", "mg_reorder_quantize_w", "mg_mixed_gemm", "mg_mixed_gemm_rows", "mg_padded_rows",
+    "mg_fused_linear",
     "mg_fused_workspace_bytes", "mg_sf_bytes", "mg_sf_offset", "mg_device_synchronize", "mg_status_string",
     "mg_measure_mfma_ceiling", "mg_calibrate_reorder_index", "mg_calibrate_workspace_bytes",
 )
@@ -43,6 +44,8 @@ def lib() -> ctypes.CDLL:
             fn = getattr(L, name)
             fn.restype, fn.argtypes = i, [p, p, i, i, i, i, i, p, p, p, p, p, p, p]
         L.mg_mixed_gemm.restype, L.mg_mixed_gemm.argtypes = i, [p] * 12 + [i] * 5 + [p, p]
+        L.mg_mixed_gemm_rows.restype, L.mg_mixed_gemm_rows.argtypes = i, [p] * 12 + [i] * 6 + [p, p]
+        L.mg_padded_rows.restype, L.mg_padded_rows.argtypes = i, [i]
         L.mg_fused_linear.restype = i
         L.mg_fused_linear.argtypes = [p] * 8 + [i] * 5 + [p, p, z, p]
         L.mg_fused_workspace_bytes.restype, L.mg_fused_workspace_bytes.argtypes = z, [i, i, i, i]
@@ -96,16 +99,35 @@ def _require(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
         raise MixedGemmError(f"{name}: expected a contiguous tensor")
 
 
+def padded_rows(m: int) -> int:
+    return int(lib().mg_padded_rows(m))
+
+
+def _rows_view(alloc_rows, rows, cols, **kw):
+    """uint8 [rows, cols] at the start of storage with room for alloc_rows rows."""
+    return torch.empty((alloc_rows, cols), **kw)[:rows]
+
+
 def alloc_quant_outputs(rows, kn, ks, ko, operand, device):
-    """The six output tensors of a reorder-quantize call (codes x3, scales x3)."""
+    """The six output tensors of a reorder-quantize call (codes x3, scales x3), with the
+    reference's shapes.  For activations the storage behind them has room for whole 256-row
+    tiles, which lets matmul() run a ragged token count on the whole-tile kernel."""
     w = operand == MG_OPERAND_B
     u8 = dict(dtype=torch.uint8, device=device)
-    return (torch.empty((rows, kn // 2), **u8),
-            torch.empty((rows, ks // 2 if w else ks // 4 * 3), **u8),
-            torch.empty((rows, ko // 2 if w else ko), **u8),
-            torch.empty(sf_bytes(rows, kn, operand), **u8),
-            torch.empty(sf_bytes(rows, ks, operand), **u8),
-            torch.empty(sf_bytes(rows, ko, operand), **u8))
+    r = rows if w else padded_rows(rows)
+
+    def sf(kseg):
+        return torch.empty(max(sf_bytes(r, kseg, operand), sf_bytes(rows, kseg, operand)), **u8)[:sf_bytes(rows, kseg, operand)]
+
+    return (_rows_view(r, rows, kn // 2, **u8),
+            _rows_view(r, rows, ks // 2 if w else ks // 4 * 3, **u8),
+            _rows_view(r, rows, ko // 2 if w else ko, **u8),
+            sf(kn), sf(ks), sf(ko))
+
+
+def _capacity(t: torch.Tensor) -> int:
+    """Bytes readable from t's first element to the end of its storage."""
+    return t.untyped_storage().nbytes() - t.storage_offset() * t.element_size()
 
 
 def _reorder_quantize(fn_name, operand, t, idx, kn, ks, ko, out=None):
@@ -143,9 +165,13 @@ def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None
     kn, ks, ko = an.shape[1] * 2, as_.shape[1] * 4 // 3, ao.shape[1]
     if out is None:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=an.device)
-    status = lib().mg_mixed_gemm(_ptr(an), _ptr(bn), _ptr(as_), _ptr(bs), _ptr(ao), _ptr(bo),
-                                 _ptr(sfan), _ptr(sfbn), _ptr(sfas), _ptr(sfbs), _ptr(sfao), _ptr(sfbo),
-                                 m, n, kn, ks, ko, _ptr(out), _stream(an))
+    # rows the activation buffers are readable for: whole tiles if every storage has the room
+    r = padded_rows(m)
+    roomy = all(_capacity(t) >= r * t.shape[1] for t in (an, as_, ao)) and all(
+        _capacity(t) >= sf_bytes(r, kseg, MG_OPERAND_A) for t, kseg in ((sfan, kn), (sfas, ks), (sfao, ko)) if kseg)
+    status = lib().mg_mixed_gemm_rows(_ptr(an), _ptr(bn), _ptr(as_), _ptr(bs), _ptr(ao), _ptr(bo),
+                                      _ptr(sfan), _ptr(sfbn), _ptr(sfas), _ptr(sfbs), _ptr(sfao), _ptr(sfbo),
+                                      m, r if roomy else m, n, kn, ks, ko, _ptr(out), _stream(an))
     check(status, "mg_mixed_gemm")
     return out
 

@@ -12,7 +12,7 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
 hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
-                             int N, int KN, int KS, int KO, void* d, hipStream_t stream);
+                             int a_rows, int N, int KN, int KS, int KO, void* d, hipStream_t stream);
 size_t calibrate_workspace_bytes(int K);
 hipError_t launch_calibrate(const void* x, int rows, int K, int16_t* idx, void* workspace, hipStream_t stream);
 }  // namespace mg
@@ -60,12 +60,12 @@ int mg_reorder_quantize_w(const void* w_bf16, const int16_t* idx, int N, int K, 
   return reorder_quantize<true>(w_bf16, idx, N, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream);
 }
 
-int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs, const uint8_t* ao,
-                  const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
-                  const uint8_t* sfao, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO, void* d_bf16,
-                  void* stream) {
+int mg_mixed_gemm_rows(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs, const uint8_t* ao,
+                       const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas,
+                       const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M, int a_rows, int N, int KN,
+                       int KS, int KO, void* d_bf16, void* stream) {
   if (int s = check_split(M, KN, KS, KO)) return s;
-  if (N < 0) return MG_ERR_BAD_SHAPE;
+  if (N < 0 || a_rows < M) return MG_ERR_BAD_SHAPE;
   if (M == 0 || N == 0) return MG_OK;
   if (!ptr_ok(d_bf16, true)) return MG_ERR_BAD_POINTER;
   if (!ptr_ok(an, KN > 0) || !ptr_ok(bn, KN > 0) || !ptr_ok(as_, KS > 0) || !ptr_ok(bs, KS > 0) ||
@@ -73,9 +73,18 @@ int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, cons
     return MG_ERR_BAD_POINTER;
   if ((KN > 0 && (!sfan || !sfbn)) || (KS > 0 && (!sfas || !sfbs)) || (KO > 0 && (!sfao || !sfbo)))
     return MG_ERR_BAD_POINTER;
-  return (int)mg::launch_mixed_gemm(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, N, KN, KS, KO, d_bf16,
-                                    static_cast<hipStream_t>(stream));
+  return (int)mg::launch_mixed_gemm(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, a_rows, N, KN, KS, KO,
+                                    d_bf16, static_cast<hipStream_t>(stream));
 }
+
+int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs, const uint8_t* ao,
+                  const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
+                  const uint8_t* sfao, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO, void* d_bf16,
+                  void* stream) {
+  return mg_mixed_gemm_rows(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, M, N, KN, KS, KO, d_bf16, stream);
+}
+
+int mg_padded_rows(int M) { return M <= 0 ? 0 : (M + 255) / 256 * 256; }
 
 size_t mg_sf_bytes(int rows, int kseg, int operand) {
   if (rows < 0 || kseg < 0) return 0;
@@ -87,11 +96,14 @@ size_t mg_sf_bytes(int rows, int kseg, int operand) {
 
 size_t mg_sf_offset(int row, int kb, int kseg) { return mg::sf_offset(row, kb, (kseg + 127) / 128); }
 
+// The quantized activations live in the workspace with room for whole 256-row tiles, so that the
+// GEMM may read (and ignore) the rows between M and the next multiple of 256.
 size_t mg_fused_workspace_bytes(int M, int KN, int KS, int KO) {
   if (M < 0 || KN < 0 || KS < 0 || KO < 0) return 0;
-  return align256((size_t)M * (KN / 2)) + align256((size_t)M * (KS / 4 * 3)) + align256((size_t)M * KO) +
-         align256(mg_sf_bytes(M, KN, MG_OPERAND_A)) + align256(mg_sf_bytes(M, KS, MG_OPERAND_A)) +
-         align256(mg_sf_bytes(M, KO, MG_OPERAND_A));
+  const int R = mg_padded_rows(M);
+  return align256((size_t)R * (KN / 2)) + align256((size_t)R * (KS / 4 * 3)) + align256((size_t)R * KO) +
+         align256(mg_sf_bytes(R, KN, MG_OPERAND_A)) + align256(mg_sf_bytes(R, KS, MG_OPERAND_A)) +
+         align256(mg_sf_bytes(R, KO, MG_OPERAND_A));
 }
 
 int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
@@ -102,15 +114,16 @@ int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, c
   if (M == 0 || N == 0) return MG_OK;
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return MG_ERR_BAD_POINTER;
   if (workspace_bytes < mg_fused_workspace_bytes(M, KN, KS, KO)) return MG_ERR_BAD_SHAPE;
+  const int R = mg_padded_rows(M);
   uint8_t* p = static_cast<uint8_t*>(workspace);
-  uint8_t* qn = p;  p += align256((size_t)M * (KN / 2));
-  uint8_t* qs = p;  p += align256((size_t)M * (KS / 4 * 3));
-  uint8_t* qo = p;  p += align256((size_t)M * KO);
-  uint8_t* sfn = p; p += align256(mg_sf_bytes(M, KN, MG_OPERAND_A));
-  uint8_t* sfs = p; p += align256(mg_sf_bytes(M, KS, MG_OPERAND_A));
+  uint8_t* qn = p;  p += align256((size_t)R * (KN / 2));
+  uint8_t* qs = p;  p += align256((size_t)R * (KS / 4 * 3));
+  uint8_t* qo = p;  p += align256((size_t)R * KO);
+  uint8_t* sfn = p; p += align256(mg_sf_bytes(R, KN, MG_OPERAND_A));
+  uint8_t* sfs = p; p += align256(mg_sf_bytes(R, KS, MG_OPERAND_A));
   uint8_t* sfo = p;
   if (int s = mg_reorder_quantize_x(x_bf16, idx, M, KN + KS + KO, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream)) return s;
-  return mg_mixed_gemm(qn, bn, qs, bs, qo, bo, sfn, sfbn, sfs, sfbs, sfo, sfbo, M, N, KN, KS, KO, d_bf16, stream);
+  return mg_mixed_gemm_rows(qn, bn, qs, bs, qo, bo, sfn, sfbn, sfs, sfbs, sfo, sfbo, M, R, N, KN, KS, KO, d_bf16, stream);
 }
 
 size_t mg_calibrate_workspace_bytes(int K) { return K > 0 ? mg::calibrate_workspace_bytes(K) : 0; }

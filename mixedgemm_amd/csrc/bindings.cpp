@@ -61,6 +61,18 @@ Tensor bytes(const Tensor& like, std::initializer_list<int64_t> shape) {
   return torch::empty(shape, torch::dtype(torch::kUInt8).device(like.device()));
 }
 
+// uint8 [rows, cols] (or [n] when cols < 0) at the start of a larger allocation: the tensor has the
+// reference's shape, its storage the room for whole 256-row tiles
+Tensor roomy(const Tensor& like, int64_t alloc, int64_t shown, int64_t cols) {
+  if (cols < 0) return bytes(like, {alloc < shown ? shown : alloc}).narrow(0, 0, shown);
+  return bytes(like, {alloc < shown ? shown : alloc, cols}).narrow(0, 0, shown);
+}
+
+// bytes readable from the tensor's first element to the end of its storage
+int64_t capacity(const Tensor& t) {
+  return static_cast<int64_t>(t.storage().nbytes()) - t.storage_offset() * static_cast<int64_t>(t.element_size());
+}
+
 Tensor matmul(const Tensor& AN, const Tensor& BN, const Tensor& AS, const Tensor& BS, const Tensor& AO, const Tensor& BO,
               const Tensor& SFAN, const Tensor& SFBN, const Tensor& SFAS, const Tensor& SFBS, const Tensor& SFAO,
               const Tensor& SFBO) {
@@ -71,11 +83,18 @@ Tensor matmul(const Tensor& AN, const Tensor& BN, const Tensor& AS, const Tensor
   const int KS = static_cast<int>(AS.size(1)) * 4 / 3;
   const int KO = static_cast<int>(AO.size(1));
   Tensor C = torch::zeros({M, N}, torch::dtype(torch::kBFloat16).device(AN.device()));
-  const int status = mg_mixed_gemm(AN.data_ptr<uint8_t>(), BN.data_ptr<uint8_t>(), AS.data_ptr<uint8_t>(),
-                                   BS.data_ptr<uint8_t>(), AO.data_ptr<uint8_t>(), BO.data_ptr<uint8_t>(),
-                                   SFAN.data_ptr<uint8_t>(), SFBN.data_ptr<uint8_t>(), SFAS.data_ptr<uint8_t>(),
-                                   SFBS.data_ptr<uint8_t>(), SFAO.data_ptr<uint8_t>(), SFBO.data_ptr<uint8_t>(), M, N, KN,
-                                   KS, KO, C.data_ptr<at::BFloat16>(), current_stream(AN));
+  // activation buffers that reorder_quantize_x of this module made have room for whole tiles
+  const int R = mg_padded_rows(M);
+  const bool room = capacity(AN) >= (int64_t)R * AN.size(1) && capacity(AS) >= (int64_t)R * AS.size(1) &&
+                    capacity(AO) >= (int64_t)R * AO.size(1) &&
+                    capacity(SFAN) >= (int64_t)mg_sf_bytes(R, KN, MG_OPERAND_A) &&
+                    capacity(SFAS) >= (int64_t)mg_sf_bytes(R, KS, MG_OPERAND_A) &&
+                    capacity(SFAO) >= (int64_t)mg_sf_bytes(R, KO, MG_OPERAND_A);
+  const int status = mg_mixed_gemm_rows(AN.data_ptr<uint8_t>(), BN.data_ptr<uint8_t>(), AS.data_ptr<uint8_t>(),
+                                        BS.data_ptr<uint8_t>(), AO.data_ptr<uint8_t>(), BO.data_ptr<uint8_t>(),
+                                        SFAN.data_ptr<uint8_t>(), SFBN.data_ptr<uint8_t>(), SFAS.data_ptr<uint8_t>(),
+                                        SFBS.data_ptr<uint8_t>(), SFAO.data_ptr<uint8_t>(), SFBO.data_ptr<uint8_t>(), M,
+                                        room ? R : M, N, KN, KS, KO, C.data_ptr<at::BFloat16>(), current_stream(AN));
   finish(status, "GEMM");
   return C;
 }
@@ -90,12 +109,13 @@ SixTensors reorder_quantize(const Tensor& T, const Tensor& reorder_index, int KN
     throw std::runtime_error(std::string("Value error in ") + what + " ");
   }
   const int operand = kWeights ? MG_OPERAND_B : MG_OPERAND_A;
-  Tensor QN = bytes(T, {rows, KN / 2});
-  Tensor QS = bytes(T, {rows, kWeights ? KS / 2 : KS / 4 * 3});
-  Tensor QO = bytes(T, {rows, kWeights ? KO / 2 : KO});
-  Tensor SFN = bytes(T, {static_cast<int64_t>(mg_sf_bytes(rows, KN, operand))});
-  Tensor SFS = bytes(T, {static_cast<int64_t>(mg_sf_bytes(rows, KS, operand))});
-  Tensor SFO = bytes(T, {static_cast<int64_t>(mg_sf_bytes(rows, KO, operand))});
+  const int R = kWeights ? rows : mg_padded_rows(rows);
+  Tensor QN = roomy(T, R, rows, KN / 2);
+  Tensor QS = roomy(T, R, rows, kWeights ? KS / 2 : KS / 4 * 3);
+  Tensor QO = roomy(T, R, rows, kWeights ? KO / 2 : KO);
+  Tensor SFN = roomy(T, static_cast<int64_t>(mg_sf_bytes(R, KN, operand)), static_cast<int64_t>(mg_sf_bytes(rows, KN, operand)), -1);
+  Tensor SFS = roomy(T, static_cast<int64_t>(mg_sf_bytes(R, KS, operand)), static_cast<int64_t>(mg_sf_bytes(rows, KS, operand)), -1);
+  Tensor SFO = roomy(T, static_cast<int64_t>(mg_sf_bytes(R, KO, operand)), static_cast<int64_t>(mg_sf_bytes(rows, KO, operand)), -1);
   auto* fn = kWeights ? &mg_reorder_quantize_w : &mg_reorder_quantize_x;
   const int status = fn(T.data_ptr<at::BFloat16>(), reorder_index.data_ptr<int16_t>(), rows, K, KN, KS, KO,
                         QN.data_ptr<uint8_t>(), QS.data_ptr<uint8_t>(), QO.data_ptr<uint8_t>(), SFN.data_ptr<uint8_t>(),

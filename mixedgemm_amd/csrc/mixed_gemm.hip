@@ -134,16 +134,16 @@ mixed_gemm_direct_kernel(const uint8_t* __restrict__ an, const uint8_t* __restri
 
 
 // ---------------------------------------------------------------------------
-// Decode kernel: M <= 16 tokens, weights streamed once (HBM-bound).
+// Skinny kernel: few tokens (decode, small batches, the ragged last rows of a
+// prefill), weights streamed once per 16 * G tokens (HBM- or L2-bound).
 //
-// A workgroup of 4 waves owns 16 output features; the K steps (128 elements
-// each, counted over the three segments) are dealt to the 4 waves in contiguous
-// quarters, so 3.5 waves per SIMD each keep all their weight loads in flight at
-// once.  Every load of a wave is issued before its first MFMA; the 4 partial
-// 16x16 tiles are summed through LDS and rounded to bf16 once.
+// A workgroup of 4 waves owns 16 output features and G groups of 16 tokens; the K
+// steps (128 elements each, counted over the three segments) are dealt to the 4
+// waves in contiguous quarters.  A wave issues every load of a round of steps
+// (weights, the G token groups, scales; addresses clamped, no branches) before
+// the round's first MFMA; the 4 partial 16x16 tiles per group are summed through
+// LDS and rounded to bf16 once.  G = 1 is the decode case.
 // ---------------------------------------------------------------------------
-constexpr int kDecodeMaxSteps = 8;   // K steps a wave keeps in flight at once
-
 struct DecodeSeg {
   const uint8_t* a;
   const uint8_t* b;
@@ -158,106 +158,137 @@ __device__ __forceinline__ v4f decode_mfma(v8i wb, v8i xa, v4f acc, int sw, int 
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wb, xa, acc, kFmtE2M1, FMT, 0, sw, 0, sx);
 }
 
+template <int G>
 __global__ void __launch_bounds__(256)
-mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N, int steps_per_wave,
+mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, int M, int N, int steps_per_wave,
                          uint16_t* __restrict__ d) {
-  __shared__ float partial[4][16 * 16];
+  constexpr int S = G >= 8 ? 1 : 8 / G;   // K steps a wave keeps in flight at once
+  __shared__ float partial[4][G][16 * 16];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, g = lane >> 4;
   const int n = blockIdx.x * 16 + i;
-  const bool n_ok = n < N, m_ok = i < M;
-  const int nc = min(n, N - 1), mc = min(i, M - 1);   // clamped rows: every load is in bounds and unconditional
+  const int m0 = m_base + blockIdx.y * (G * 16) + i;      // this lane's token in group 0
+  const bool n_ok = n < N;
+  const int nc = min(n, N - 1);   // clamped rows: every load is in bounds and unconditional
   const int total = s4.steps + s6.steps + s8.steps;
-  v4f acc = {0.f, 0.f, 0.f, 0.f};
-
-  for (int r0 = 0; r0 < steps_per_wave; r0 += kDecodeMaxSteps) {
-  const int t0 = wave * steps_per_wave + r0, t_end = min(total, wave * steps_per_wave + steps_per_wave);
-
-  // Straight-line issue of every load of this wave (addresses clamped, no
-  // branches), so all of them are in flight together; masking comes afterwards.
-  v4i wq[kDecodeMaxSteps], xa[kDecodeMaxSteps], xb[kDecodeMaxSteps];
-  int sw[kDecodeMaxSteps], sx[kDecodeMaxSteps];
+  v4f acc[G];
 #pragma unroll
-  for (int k = 0; k < kDecodeMaxSteps; ++k) {
-    const int t = min(t0 + k, total - 1);
-    const int seg = t < s4.steps ? 0 : (t < s4.steps + s6.steps ? 1 : 2);
-    const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
-    const uint8_t* pa = seg == 0 ? s4.a : (seg == 1 ? s6.a : s8.a);
-    const uint8_t* pb = seg == 0 ? s4.b : (seg == 1 ? s6.b : s8.b);
-    const uint8_t* psa = seg == 0 ? s4.sfa : (seg == 1 ? s6.sfa : s8.sfa);
-    const uint8_t* psb = seg == 0 ? s4.sfb : (seg == 1 ? s6.sfb : s8.sfb);
-    const int nblk = seg == 0 ? s4.nblk : (seg == 1 ? s6.nblk : s8.nblk);
-    const int katoms = seg == 0 ? s4.steps : (seg == 1 ? s6.steps : s8.steps);
-    const int xbytes = seg == 0 ? 16 : (seg == 1 ? 24 : 32);   // activation bytes per 32-element block
-    const int left = nblk - 4 * q;
-    const int gc = min(g, left - 1);
-    wq[k] = *reinterpret_cast<const v4i*>(pb + (size_t)nc * nblk * 16 + q * 64 + gc * 16);
-    // activations: two 16-byte pieces.  E2M1: block g (second piece unused);
-    // E3M2: bytes [0,16) and [8,24) of block g; E4M3: K [16g,+16) and [64+16g,+16).
-    const uint8_t* xrow = pa + (size_t)mc * nblk * xbytes + q * 4 * xbytes;
-    const int a_blk = seg == 2 ? (g >> 1) : g, b_blk = seg == 2 ? 2 + (g >> 1) : g;
-    int off_a = seg == 1 ? g * 24 : g * 16;
-    int off_b = seg == 0 ? g * 16 : (seg == 1 ? g * 24 + 8 : 64 + g * 16);
-    off_a = a_blk < left ? off_a : 0;
-    off_b = b_blk < left ? off_b : 0;
-    xa[k] = *reinterpret_cast<const v4i*>(xrow + off_a);
-    xb[k] = *reinterpret_cast<const v4i*>(xrow + off_b);
-    sw[k] = psb[sf_offset(nc, 4 * q + gc, katoms)];
-    sx[k] = psa[sf_offset(mc, 4 * q + gc, katoms)];
-  }
+  for (int gi = 0; gi < G; ++gi) acc[gi] = v4f{0.f, 0.f, 0.f, 0.f};
 
+  for (int r0 = 0; r0 < steps_per_wave; r0 += S) {
+    const int t0 = wave * steps_per_wave + r0, t_end = min(total, wave * steps_per_wave + steps_per_wave);
+
+    // Straight-line issue of every load of this round, so all of them are in
+    // flight together; masking comes afterwards.
+    v4i wq[S], xa[S][G], xb[S][G];
+    int sw[S], sx[S][G];
 #pragma unroll
-  for (int k = 0; k < kDecodeMaxSteps; ++k) {
-    const int t = t0 + k;
-    if (t < t_end) {   // wave-uniform
+    for (int k = 0; k < S; ++k) {
+      const int t = min(t0 + k, total - 1);
       const int seg = t < s4.steps ? 0 : (t < s4.steps + s6.steps ? 1 : 2);
       const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
+      const uint8_t* pa = seg == 0 ? s4.a : (seg == 1 ? s6.a : s8.a);
+      const uint8_t* pb = seg == 0 ? s4.b : (seg == 1 ? s6.b : s8.b);
+      const uint8_t* psa = seg == 0 ? s4.sfa : (seg == 1 ? s6.sfa : s8.sfa);
+      const uint8_t* psb = seg == 0 ? s4.sfb : (seg == 1 ? s6.sfb : s8.sfb);
       const int nblk = seg == 0 ? s4.nblk : (seg == 1 ? s6.nblk : s8.nblk);
+      const int katoms = seg == 0 ? s4.steps : (seg == 1 ? s6.steps : s8.steps);
+      const int xbytes = seg == 0 ? 16 : (seg == 1 ? 24 : 32);   // activation bytes per 32-element block
       const int left = nblk - 4 * q;
-      const bool blk_ok = g < left;
-      const bool w_ok = n_ok && blk_ok;
-      const v4i z = {0, 0, 0, 0};
-      const v4i w4 = w_ok ? wq[k] : z;
-      const v8i wf = {w4[0], w4[1], w4[2], w4[3], 0, 0, 0, 0};
-      const int s_w = w_ok ? sw[k] : 127;
-      const int s_x = (m_ok && blk_ok) ? sx[k] : 127;
-      if (seg == 0) {
-        const v4i a4 = (m_ok && blk_ok) ? xa[k] : z;
-        const v8i xf = {a4[0], a4[1], a4[2], a4[3], 0, 0, 0, 0};
-        acc = decode_mfma<kFmtE2M1>(wf, xf, acc, s_w, s_x);
-      } else if (seg == 1) {
-        const v4i a4 = (m_ok && blk_ok) ? xa[k] : z;
-        const v4i b4 = (m_ok && blk_ok) ? xb[k] : z;
-        const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4[2], b4[3], 0, 0};
-        acc = decode_mfma<kFmtE3M2>(wf, xf, acc, s_w, s_x);
-      } else {
-        const v4i a4 = (m_ok && (g >> 1) < left) ? xa[k] : z;
-        const v4i b4 = (m_ok && 2 + (g >> 1) < left) ? xb[k] : z;
-        const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4[0], b4[1], b4[2], b4[3]};
-        acc = decode_mfma<kFmtE4M3>(wf, xf, acc, s_w, s_x);
+      const int gc = min(g, left - 1);
+      wq[k] = *reinterpret_cast<const v4i*>(pb + (size_t)nc * nblk * 16 + q * 64 + gc * 16);
+      sw[k] = psb[sf_offset(nc, 4 * q + gc, katoms)];
+      // activations: two 16-byte pieces.  E2M1: block g (second piece unused);
+      // E3M2: bytes [0,16) and [8,24) of block g; E4M3: K [16g,+16) and [64+16g,+16).
+      const int a_blk = seg == 2 ? (g >> 1) : g, b_blk = seg == 2 ? 2 + (g >> 1) : g;
+      int off_a = seg == 1 ? g * 24 : g * 16;
+      int off_b = seg == 0 ? g * 16 : (seg == 1 ? g * 24 + 8 : 64 + g * 16);
+      off_a = a_blk < left ? off_a : 0;
+      off_b = b_blk < left ? off_b : 0;
+#pragma unroll
+      for (int gi = 0; gi < G; ++gi) {
+        const int mc = min(m0 + gi * 16, M - 1);
+        const uint8_t* xrow = pa + (size_t)mc * nblk * xbytes + q * 4 * xbytes;
+        xa[k][gi] = *reinterpret_cast<const v4i*>(xrow + off_a);
+        xb[k][gi] = *reinterpret_cast<const v4i*>(xrow + off_b);
+        sx[k][gi] = psa[sf_offset(mc, 4 * q + gc, katoms)];
+      }
+    }
+
+#pragma unroll
+    for (int k = 0; k < S; ++k) {
+      const int t = t0 + k;
+      if (t < t_end) {   // wave-uniform
+        const int seg = t < s4.steps ? 0 : (t < s4.steps + s6.steps ? 1 : 2);
+        const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
+        const int nblk = seg == 0 ? s4.nblk : (seg == 1 ? s6.nblk : s8.nblk);
+        const int left = nblk - 4 * q;
+        const bool blk_ok = g < left;
+        const bool w_ok = n_ok && blk_ok;
+        const v4i z = {0, 0, 0, 0};
+        const v4i w4 = w_ok ? wq[k] : z;
+        const v8i wf = {w4[0], w4[1], w4[2], w4[3], 0, 0, 0, 0};
+        const int s_w = w_ok ? sw[k] : 127;
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi) {
+          const bool m_ok = m0 + gi * 16 < M;
+          const int s_x = (m_ok && blk_ok) ? sx[k][gi] : 127;
+          if (seg == 0) {
+            const v4i a4 = (m_ok && blk_ok) ? xa[k][gi] : z;
+            const v8i xf = {a4[0], a4[1], a4[2], a4[3], 0, 0, 0, 0};
+            acc[gi] = decode_mfma<kFmtE2M1>(wf, xf, acc[gi], s_w, s_x);
+          } else if (seg == 1) {
+            const v4i a4 = (m_ok && blk_ok) ? xa[k][gi] : z;
+            const v4i b4 = (m_ok && blk_ok) ? xb[k][gi] : z;
+            const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4[2], b4[3], 0, 0};
+            acc[gi] = decode_mfma<kFmtE3M2>(wf, xf, acc[gi], s_w, s_x);
+          } else {
+            const v4i a4 = (m_ok && (g >> 1) < left) ? xa[k][gi] : z;
+            const v4i b4 = (m_ok && 2 + (g >> 1) < left) ? xb[k][gi] : z;
+            const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4[0], b4[1], b4[2], b4[3]};
+            acc[gi] = decode_mfma<kFmtE4M3>(wf, xf, acc[gi], s_w, s_x);
+          }
+        }
       }
     }
   }
-  }
 
   // result tile is D^T: lane holds token m = lane % 16, features 4 * (lane / 16) + v
-  *reinterpret_cast<v4f*>(&partial[wave][lane * 4]) = acc;
-  __syncthreads();
-  if (wave == 0) {
-    v4f sum = acc;
 #pragma unroll
-    for (int w = 1; w < 4; ++w) {
-      const v4f p = *reinterpret_cast<const v4f*>(&partial[w][lane * 4]);
-      sum += p;
-    }
+  for (int gi = 0; gi < G; ++gi) *reinterpret_cast<v4f*>(&partial[wave][gi][lane * 4]) = acc[gi];
+  __syncthreads();
+  // wave w sums and writes groups w, w + 4, ...
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) {
+    if ((gi & 3) != wave && G >= 4) continue;
+    if (G < 4 && wave != gi) continue;
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) sum += *reinterpret_cast<const v4f*>(&partial[w][gi][lane * 4]);
     const int nn = blockIdx.x * 16 + 4 * g;
-    if (m_ok) {
-      uint16_t* dst = d + (size_t)i * N + nn;
+    const int m = m0 + gi * 16;
+    if (m < M) {
+      uint16_t* dst = d + (size_t)m * N + nn;
 #pragma unroll
       for (int v = 0; v < 4; ++v)
         if (nn + v < N) dst[v] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
     }
   }
+}
+
+hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int m_base, int M, int N,
+                         uint16_t* d, hipStream_t stream) {
+  const int rows = M - m_base;
+  const int steps_per_wave = (d4.steps + d6.steps + d8.steps + 3) / 4;
+  const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
+  const dim3 grid(ceil_div(N, 16), ceil_div(rows, 16 * g));
+  switch (g) {
+    case 1: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<1>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, d); break;
+    case 2: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<2>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, d); break;
+    case 4: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<4>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, d); break;
+    default: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<8>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, d); break;
+  }
+  return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------
@@ -550,23 +581,46 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO);
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
-                                 int M, int N, int KN, int KS, int KO, void* d, hipStream_t stream);
+                                 int M, int m_store, int N, int KN, int KS, int KO, void* d, hipStream_t stream);
 
+// Rough launch times in microseconds (measured on MI355X, K = 4096: a 128-wide stage takes ~1.05 us
+// with every CU busy and ~0.7 us when at most half of them are, plus ~8 us of fill and drain per
+// round of 256 tiles; 0.28 ns per 16 tokens x 16 features x 128 K on the skinny kernel), only to
+// choose between the two for fewer than 256 tokens.
+static double pipelined_us(int m_pad, int N, int stages) {
+  const int tiles = (m_pad / 256) * (N / 256);
+  return (double)((tiles + 255) / 256) * (stages * (tiles <= 128 ? 0.7 : 1.05) + 8.0);
+}
+static double skinny_us(int rows, int N, int steps) {
+  return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * 0.28e-3;
+}
+
+// a_rows: token rows for which the activation codes and scales are readable (>= M)
 hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
-                             int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
+                             int a_rows, int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
   if (M == 0 || N == 0) return hipSuccess;
-  if (mixed_gemm_256_supported(M, N, KN, KS, KO))
-    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, N, KN, KS, KO, d, stream);
-  if (M <= 16) {
-    const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
-    const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
-    const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};
-    const int steps_per_wave = (d4.steps + d6.steps + d8.steps + 3) / 4;
-    hipLaunchKernelGGL(mixed_gemm_decode_kernel, dim3(ceil_div(N, 16)), dim3(256), 0, stream, d4, d6, d8, M, N,
-                       steps_per_wave, static_cast<uint16_t*>(d));
-    return hipGetLastError();
+  const int m_pad = (M + 255) / 256 * 256;
+  const int steps = (KN + 127) / 128 + (KS + 127) / 128 + (KO + 127) / 128;
+  // whole 256-row tiles, the last one possibly reading rows past M (readable up to a_rows) and
+  // not writing them
+  if ((M == m_pad || a_rows >= m_pad) && mixed_gemm_256_supported(m_pad, N, KN, KS, KO) &&
+      (M >= 256 || pipelined_us(m_pad, N, steps) < skinny_us(M, N, steps)))
+    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_pad, M, N, KN, KS, KO, d,
+                                 stream);
+  const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
+  const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
+  const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};
+  if (M < 256 && KN + KS + KO > 0) return launch_skinny(d4, d6, d8, 0, M, N, static_cast<uint16_t*>(d), stream);
+  // ragged token count: whole 256-row tiles on the pipelined kernel (same pointers: rows are
+  // independent and a scale atom never spans a 256-row boundary), the last rows on the skinny one
+  const int m_main = M / 256 * 256;
+  if (m_main < M && mixed_gemm_256_supported(m_main, N, KN, KS, KO)) {
+    hipError_t e = launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_main, m_main, N, KN,
+                                         KS, KO, d, stream);
+    if (e != hipSuccess) return e;
+    return launch_skinny(d4, d6, d8, m_main, M, N, static_cast<uint16_t*>(d), stream);
   }
   // the tiled kernel needs whole tiles and whole 128-wide K stages
   if (M % kTileM == 0 && N % kTileN == 0 && KN % kStageK == 0 && KS % kStageK == 0 && KO % kStageK == 0 &&

@@ -659,7 +659,7 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
 // REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.
 template <bool REGULAR, bool REM>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ d) {
+mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
   Plan plan;
   plan.a0 = uni(plan_arg.a0); plan.a1 = uni(plan_arg.a1); plan.a2 = uni(plan_arg.a2);
@@ -785,10 +785,11 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, uint16_t* __restrict__ 
     const int r = c.lane >> 4, cc = c.lane & 15;
     const uint8_t* rd = stage + r * kPitch + cc * 16;
     uint16_t* out = d + (size_t)(c.m0 + c.wm * 128 + r) * N + c.n0 + c.wn * 128 + cc * 8;
+    const int rows_left = m_store - (c.m0 + c.wm * 128 + r);   // token rows at or past m_store are not written
 #pragma unroll 8
     for (int i = 0; i < 32; ++i) {
       const v4u v = *reinterpret_cast<const v4u*>(rd + i * 4 * kPitch);
-      *reinterpret_cast<v4u*>(out + (size_t)i * 4 * N) = v;
+      if (i * 4 < rows_left) *reinterpret_cast<v4u*>(out + (size_t)i * 4 * N) = v;
     }
   }
 }
@@ -806,11 +807,11 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
-                                 int M, int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
+                                 int M, int m_store, int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
   // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
   const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
   const bool rem = (KN | KS | KO) % 128 != 0;
-  typedef void (*kernel_t)(Plan, int, int, uint16_t*);
+  typedef void (*kernel_t)(Plan, int, int, int, uint16_t*);
   const kernel_t kernels[2][2] = {{mixed_gemm_256_kernel<false, false>, mixed_gemm_256_kernel<false, true>},
                                   {mixed_gemm_256_kernel<true, false>, mixed_gemm_256_kernel<true, true>}};
   const kernel_t kernel = kernels[regular][rem];
@@ -830,7 +831,7 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.blk0 = KN / 32; p.blk1 = KS / 32; p.blk2 = KO / 32;
   p.total = p.st0 + p.st1 + p.st2;
   const int tiles_n = N / kT, tiles_m = M / kT;
-  hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage, stream, p, tiles_n, N,
+  hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store,
                      static_cast<uint16_t*>(d));
   return hipGetLastError();
 }

@@ -169,6 +169,13 @@ GEMM_SHAPES = [
     (256, 256, 384, 384, 384), (512, 256, 512, 384, 128), (256, 512, 384, 512, 256),
     # segments that end 32, 64 or 96 elements past their last whole 128-wide stage
     (256, 256, 448, 416, 224), (256, 512, 2240, 1248, 448), (512, 256, 160, 480, 352),
+    # skinny kernel with 2, 4 and 8 token groups: ragged M and N, partial K steps, an empty segment
+    (17, 48, 256, 128, 128), (32, 200, 96, 160, 64), (50, 40, 2560, 1408, 128), (64, 64, 0, 4928, 448),
+    (100, 256, 448, 224, 64), (128, 4096, 2560, 1408, 128), (255, 272, 128, 128, 128), (200, 1000, 640, 256, 256),
+    # ragged token count: whole 256-row tiles on the pipelined kernel + the last rows on the skinny one
+    (300, 512, 2560, 1408, 128), (257, 256, 384, 384, 384), (767, 256, 448, 416, 224),
+    # 256 or more tokens with an empty segment: the LDS-tiled kernel
+    (256, 256, 256, 0, 0), (384, 256, 0, 256, 128), (256, 512, 128, 0, 128),
 ]
 
 
@@ -225,8 +232,14 @@ def test_gemm_operand_bit_order_one_hot(abi, seg):
         np.testing.assert_array_equal(d.float().cpu().numpy(), want, err_msg=f"{seg} trial {trial} row {row} k {kk}")
 
 
-def test_fused_linear_equals_quantize_then_gemm(abi):
-    m, n, kn, ks, ko = 96, 256, 2560, 1408, 128
+@pytest.mark.parametrize("m,n,kn,ks,ko", [
+    (96, 256, 2560, 1408, 128),
+    # ragged token counts: the last 256-row tile reads rows past M from the padded buffers and does not write them
+    (300, 512, 2560, 1408, 128), (130, 2560, 384, 384, 384), (1000, 256, 448, 416, 224), (255, 4096, 2560, 896, 128),
+    (70, 14336, 2560, 1408, 128),
+])
+def test_fused_linear_equals_quantize_then_gemm(abi, m, n, kn, ks, ko):
+    _say("fused", m, n, kn, ks, ko)
     k = kn + ks + ko
     x = H.make_activations(m, k, 50)
     w = H.make_weights(n, k, 51)
@@ -236,10 +249,14 @@ def test_fused_linear_equals_quantize_then_gemm(abi):
     aq = abi.reorder_quantize_x(xd, idd, kn, ks, ko)
     d1 = abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5])
     d2 = abi.fused_linear(xd, idd, bq[0], bq[1], bq[2], bq[3], bq[4], bq[5], kn, ks, ko)
+    # exact-size activation buffers (no room past M): whole tiles + the skinny kernel for the last rows
+    tight = [t.clone() for t in aq]
+    d3 = abi.matmul(tight[0], bq[0], tight[1], bq[1], tight[2], bq[2], tight[3], bq[3], tight[4], bq[4], tight[5], bq[5])
     torch.cuda.synchronize()
     assert torch.equal(d1, d2)
     qx, qw = _oracle_operands(x, w, idx, kn, ks, ko)
     _check_gemm(d2, qx, qw, "fused")
+    _check_gemm(d3, qx, qw, "exact-size buffers")
 
 
 def test_config0_end_to_end(abi):

@@ -34,9 +34,10 @@ P46, P8 = 10100.0, 5000.0
 # counter's reading for `bench.py --calibrate-copy`; None where not measured.  The figures and the
 # commands are in profiles/.
 MEASURED_TRAFFIC = {
-    "gemm_c3": int((154367.6 * 1.9998 + 149632.0 * 1.0) * 1024),   # L2 misses re-read operands ~7x; D written once (+27 %)
-    "quant_c1": int((16453.1 * 1.9998 + 10880.1 * 1.0) * 1024),    # 44.9 MB against 44.2 MB algorithmic
-    "decode_c2": int((18122.4 * 1.9998 + 224.0 * 1.0) * 1024),     # 37.3 MB against 31.4 MB algorithmic
+    "gemm_c3": int((137925.4 * 1.99981 + 118272.0 * 1.0) * 1024),   # L2 misses re-read operands ~7x; D written once (+3 %)
+    "quant_c1": int((16455.2 * 1.99981 + 10883.8 * 1.0) * 1024),    # 44.8 MB against 44.2 MB algorithmic
+    "decode_c2": int((18141.1 * 1.99981 + 224.0 * 1.0) * 1024),     # 37.4 MB against 31.4 MB algorithmic
+    "calibrate_c1": int(((16413.1 + 1038.8 + 81.5) * 1.99981 + (2048.0 + 16.0 + 56.3) * 1.0) * 1024),   # three kernels
 }
 
 
@@ -184,7 +185,8 @@ def main():
             "workload": "reorder index of the c1 activations: per-channel absmax over M=4096 rows + sort of K=4096 channels",
             "value": round(cb / (c_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "avg_ms": round(c_ms, 5),
             "roofline": {"bound": "hbm", "achieved": round(cb / (c_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(cb / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": cb},
+                         "frac": round(cb / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("calibrate_c1"),
+                         "algorithmic_bytes": cb},
         }
         del xs, outs, base
 

@@ -92,8 +92,8 @@ def graph_ms(launch, iters, warmup=3, repeats=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -131,7 +131,9 @@ def main():
     w = H.make_weights(n, k, 2234 + 3)
     idx = H.absmax_sort_index(x)
     xd, wd, idd = x.to(dev), w.to(dev), idx.to(dev)
+    # weights: quantized and put in tile-major order once, outside the timed region (the offline pack)
     bq = abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+    bt = abi.tile_weights(*bq[:3])
     aq = abi.alloc_quant_outputs(m, kn, ks, ko, abi.MG_OPERAND_A, dev)
     d = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
     torch.cuda.synchronize()
@@ -142,7 +144,7 @@ def main():
         abi.reorder_quantize_x(xd, idd, kn, ks, ko, out=aq)
         if pair:
             pair[0].record()
-        abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], out=d)
+        abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], out=d, w_tiled=True)
         if pair:
             pair[1].record()
 
@@ -168,6 +170,19 @@ def main():
 
     extra = {}
     if not args.no_extra:
+        # ------------------------------------------------------------ c3 GEMM with the weights as reorder_quantize_w leaves them
+        rm, tl = [], []
+        for _ in range(5):   # alternate: the chip's clock drifts with load, medians of interleaved runs compare fairly
+            rm.append(graph_ms(lambda i: abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4],
+                                                    aq[5], bq[5], out=d), 20, repeats=2))
+            tl.append(graph_ms(lambda i: abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4],
+                                                    aq[5], bq[5], out=d, w_tiled=True), 20, repeats=2))
+        rm_ms, tl_ms = sorted(rm)[2], sorted(tl)[2]
+        extra["gemm_c3_weight_layouts"] = {
+            "note": "c3 GEMM alone, 20 launches replayed as a HIP graph (no host launch gaps), median of 5 interleaved runs",
+            "row_major_runs_ms": [round(v, 5) for v in rm], "tile_major_runs_ms": [round(v, 5) for v in tl],
+            "row_major_ms": round(rm_ms, 5), "row_major_tflops": round(flops / (rm_ms * 1e-3) / 1e12, 1),
+            "tile_major_ms": round(tl_ms, 5), "tile_major_tflops": round(flops / (tl_ms * 1e-3) / 1e12, 1)}
         # ------------------------------------------------------------ c1: reorder-quantize alone, HBM-bound
         m1, _, k1, kn1, ks1, ko1 = H.CONFIGS["c1"]
         nsets = 8                                    # 8 x 44 MB > 256 MB Infinity Cache
@@ -246,6 +261,9 @@ def main():
             xm = H.make_activations(mm, kk, 1234 + 4, student_t=(tag == "c4")).to(dev)
             idm = abi.calibrate_reorder_index(xm)
             wqm = abi.reorder_quantize_w(H.make_weights(nn, kk, 2234 + 4).to(dev), idm, knm, ksm, kom)
+            tiled = abi.weights_tileable(nn, knm, ksm, kom)
+            if tiled:
+                wqm = abi.tile_weights(*wqm[:3]) + wqm[3:]
             aqm = abi.alloc_quant_outputs(mm, knm, ksm, kom, abi.MG_OPERAND_A, dev)
             dm = torch.empty((mm, nn), dtype=torch.bfloat16, device=dev)
 
@@ -253,11 +271,12 @@ def main():
                 abi.reorder_quantize_x(xm, idm, knm, ksm, kom, out=aqm)
 
             def gemm():
-                abi.matmul(aqm[0], wqm[0], aqm[1], wqm[1], aqm[2], wqm[2], aqm[3], wqm[3], aqm[4], wqm[4], aqm[5], wqm[5], out=dm)
+                abi.matmul(aqm[0], wqm[0], aqm[1], wqm[1], aqm[2], wqm[2], aqm[3], wqm[3], aqm[4], wqm[4], aqm[5], wqm[5], out=dm,
+                           w_tiled=tiled)
 
             times = [graph_ms(lambda i: quant(), 20), graph_ms(lambda i: gemm(), 20)]
             flops = 2.0 * mm * nn * kk
-            matrix.append({"config": tag, "M": mm, "N": nn, "K": kk, "split": [knm, ksm, kom],
+            matrix.append({"config": tag, "M": mm, "N": nn, "K": kk, "split": [knm, ksm, kom], "weights_tiled": bool(tiled),
                            "quant_ms": round(times[0], 5), "gemm_ms": round(times[1], 5),
                            "gemm_tflops": round(flops / (times[1] * 1e-3) / 1e12, 1),
                            "fused_tflops": round(flops / ((times[0] + times[1]) * 1e-3) / 1e12, 1),
@@ -265,6 +284,23 @@ def main():
             del xm, wqm, aqm, dm
         extra["shape_matrix"] = {"note": "back-to-back launches on one buffer set (operands may sit in the 256 MB "
                                          "Infinity Cache); 20 launches per kernel replayed as a HIP graph, 3 replays", "rows": matrix}
+
+        # ------------------------------------------------------------ one activation format at a time (c3's M, N, K)
+        # the 256x256 kernel needs all three segments, so the other two get one 128-wide stage each
+        per_format = []
+        for name, (knf, ksf, kof) in (("e2m1", (3840, 128, 128)), ("e3m2", (128, 3840, 128)), ("e4m3", (128, 128, 3840))):
+            aqf = abi.reorder_quantize_x(xd, idd, knf, ksf, kof)
+            wqf = abi.reorder_quantize_w(wd, idd, knf, ksf, kof)
+            df = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            f_ms = graph_ms(lambda i: abi.matmul(aqf[0], wqf[0], aqf[1], wqf[1], aqf[2], wqf[2], aqf[3], wqf[3],
+                                                 aqf[4], wqf[4], aqf[5], wqf[5], out=df), 20)
+            pk = blended_peak(knf, ksf, kof)
+            tf = 2.0 * m * n * k / (f_ms * 1e-3) / 1e12
+            per_format.append({"activations": name, "split": [knf, ksf, kof], "gemm_ms": round(f_ms, 5),
+                               "tflops": round(tf, 1), "peak": round(pk, 1), "frac": round(tf / pk, 4)})
+            del aqf, wqf, df
+        extra["per_format_gemm"] = {"note": "c3's M, N and K with 3840 of the 4096 channels in one activation format; "
+                                            "peak = the same blended nominal formula", "rows": per_format}
 
         # ------------------------------------------------------------ what the matrix cores sustain on this box
         # register-resident scaled-MFMA loop on all CUs: with pseudo-random operand bits the chip hits its
@@ -333,7 +369,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "mxfp4/mxfp6/mxfp8 x mxfp4 -> f32 accumulate -> bf16", "data": "synthetic",
         "config": {"workload": "c3 prefill: reorder-quantize bf16 X[4096,4096] + mixed GEMM vs MXFP4 W[14336,4096] "
-                               "(K split 2560 fp4 / 1408 fp6 / 128 fp8), bf16 out",
+                               "(K split 2560 fp4 / 1408 fp6 / 128 fp8), bf16 out; weight codes packed tile-major offline",
                    "M": m, "N": n, "K": k, "KN": kn, "KS": ks, "KO": ko},
         "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
     }

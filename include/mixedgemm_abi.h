@@ -74,18 +74,30 @@ int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, cons
                   int M, int N, int KN, int KS, int KO, void* d_bf16, void* stream);
 
 /*
- * The same GEMM for a caller whose activation buffers have room for more token rows than M:
- * an, as_, ao are readable for a_rows >= M rows and sfan, sfas, sfao for
- * mg_sf_bytes(a_rows, kseg, MG_OPERAND_A) bytes (what lies past row M is never used for a result).
- * With a_rows >= mg_padded_rows(M) a token count that is not a multiple of 256 runs on the
- * whole-tile kernel like any other; with a_rows == M this is mg_mixed_gemm.  The reference has
- * no counterpart: its CUTLASS GEMMs (src/fp4.cu:164-182) predicate partial tiles themselves.
+ * The same GEMM with two things a caller may know about its buffers:
+ *   a_rows -- an, as_, ao are readable for a_rows >= M token rows and sfan, sfas, sfao for
+ *     mg_sf_bytes(a_rows, kseg, MG_OPERAND_A) bytes (what lies past row M is never used for a
+ *     result).  With a_rows >= mg_padded_rows(M) a token count that is not a multiple of 256 runs on
+ *     the whole-tile kernel like any other; a_rows == M is always valid.
+ *   flags  -- MG_FLAG_W_TILED: bn, bs, bo hold the codes in the tile-major order mg_tile_weights
+ *     writes (same sizes; mg_weights_tileable(N, KN, KS, KO) must hold).  The prefill kernel's copies
+ *     then read consecutive kilobytes, which is worth 10-15 % of its time.
+ * mg_mixed_gemm is this with a_rows = M, flags = 0.  The reference has no counterpart: its CUTLASS
+ * GEMMs (src/fp4.cu:164-182) predicate partial tiles themselves and fix their operand layouts.
  */
-int mg_mixed_gemm_rows(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
-                       const uint8_t* ao, const uint8_t* bo,
-                       const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
-                       const uint8_t* sfao, const uint8_t* sfbo,
-                       int M, int a_rows, int N, int KN, int KS, int KO, void* d_bf16, void* stream);
+#define MG_FLAG_W_TILED 1u
+int mg_mixed_gemm_ex(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
+                     const uint8_t* ao, const uint8_t* bo,
+                     const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
+                     const uint8_t* sfao, const uint8_t* sfbo,
+                     int M, int a_rows, int N, int KN, int KS, int KO, unsigned flags, void* d_bf16, void* stream);
+/* Rewrites one segment's weight codes src[N, kseg/2] (row-major, as mg_reorder_quantize_w wrote them;
+ * the weight path of src/bindings.cpp:188-305) into tile-major order in dst (same size, dst != src):
+ * per 256-feature tile and 128-wide K stage one block of 16 KB, ordered as the prefill kernel stages
+ * it.  N a multiple of 256, kseg a multiple of 128.  Done once per layer, offline. */
+int mg_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, void* stream);
+/* 1 when weights of this shape can be tiled: N a multiple of 256, every segment a multiple of 128, none empty. */
+int mg_weights_tileable(int N, int KN, int KS, int KO);
 /* M rounded up to whole 256-token tiles. */
 int mg_padded_rows(int M);
 
@@ -101,6 +113,12 @@ int mg_fused_linear(const void* x_bf16, const int16_t* idx,
                     const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo,
                     int M, int N, int KN, int KS, int KO,
                     void* d_bf16, void* workspace, size_t workspace_bytes, void* stream);
+/* mg_fused_linear with the flags of mg_mixed_gemm_ex (MG_FLAG_W_TILED). */
+int mg_fused_linear_ex(const void* x_bf16, const int16_t* idx,
+                       const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                       const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo,
+                       int M, int N, int KN, int KS, int KO, unsigned flags,
+                       void* d_bf16, void* workspace, size_t workspace_bytes, void* stream);
 size_t mg_fused_workspace_bytes(int M, int KN, int KS, int KO);
 
 /* Size in bytes of one segment's scale buffer (src/bindings.cpp:91-93, 210-212);

@@ -16,9 +16,11 @@ LIB_PATH = os.path.join(_PKG, "lib", "libmixedgemm_hip.so")
 
 MG_OPERAND_A = 0
 MG_OPERAND_B = 1
+MG_FLAG_W_TILED = 1
 
 SYMBOLS = (
-    "mg_reorder_quantize_x", "mg_reorder_quantize_w", "mg_mixed_gemm", "mg_mixed_gemm_rows", "mg_padded_rows",
+    "mg_reorder_quantize_x", "mg_reorder_quantize_w", "mg_mixed_gemm", "mg_mixed_gemm_ex", "mg_padded_rows", "mg_tile_weights",
+    "mg_weights_tileable", "mg_fused_linear_ex",
     "mg_fused_linear",
     "mg_fused_workspace_bytes", "mg_sf_bytes", "mg_sf_offset", "mg_device_synchronize", "mg_status_string",
     "mg_measure_mfma_ceiling", "mg_calibrate_reorder_index", "mg_calibrate_workspace_bytes",
@@ -44,7 +46,12 @@ def lib() -> ctypes.CDLL:
             fn = getattr(L, name)
             fn.restype, fn.argtypes = i, [p, p, i, i, i, i, i, p, p, p, p, p, p, p]
         L.mg_mixed_gemm.restype, L.mg_mixed_gemm.argtypes = i, [p] * 12 + [i] * 5 + [p, p]
-        L.mg_mixed_gemm_rows.restype, L.mg_mixed_gemm_rows.argtypes = i, [p] * 12 + [i] * 6 + [p, p]
+        u = ctypes.c_uint
+        L.mg_mixed_gemm_ex.restype, L.mg_mixed_gemm_ex.argtypes = i, [p] * 12 + [i] * 6 + [u, p, p]
+        L.mg_tile_weights.restype, L.mg_tile_weights.argtypes = i, [p, p, i, i, p]
+        L.mg_weights_tileable.restype, L.mg_weights_tileable.argtypes = i, [i, i, i, i]
+        L.mg_fused_linear_ex.restype = i
+        L.mg_fused_linear_ex.argtypes = [p] * 8 + [i] * 5 + [u, p, p, z, p]
         L.mg_padded_rows.restype, L.mg_padded_rows.argtypes = i, [i]
         L.mg_fused_linear.restype = i
         L.mg_fused_linear.argtypes = [p] * 8 + [i] * 5 + [p, p, z, p]
@@ -156,8 +163,9 @@ def reorder_quantize_w(w, reorder_index, kn, ks, ko, out=None):
     return _reorder_quantize("mg_reorder_quantize_w", MG_OPERAND_B, w, reorder_index, kn, ks, ko, out)
 
 
-def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None):
-    """bf16 [M, N]; shapes are recovered from the packed operands."""
+def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None, w_tiled=False):
+    """bf16 [M, N]; shapes are recovered from the packed operands.  w_tiled: bn, bs, bo are in the
+    tile-major order of tile_weights()."""
     for name, t in (("AN", an), ("BN", bn), ("AS", as_), ("BS", bs), ("AO", ao), ("BO", bo),
                     ("SFAN", sfan), ("SFBN", sfbn), ("SFAS", sfas), ("SFBS", sfbs), ("SFAO", sfao), ("SFBO", sfbo)):
         _require(t, torch.uint8, name)
@@ -169,14 +177,15 @@ def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None
     r = padded_rows(m)
     roomy = all(_capacity(t) >= r * t.shape[1] for t in (an, as_, ao)) and all(
         _capacity(t) >= sf_bytes(r, kseg, MG_OPERAND_A) for t, kseg in ((sfan, kn), (sfas, ks), (sfao, ko)) if kseg)
-    status = lib().mg_mixed_gemm_rows(_ptr(an), _ptr(bn), _ptr(as_), _ptr(bs), _ptr(ao), _ptr(bo),
-                                      _ptr(sfan), _ptr(sfbn), _ptr(sfas), _ptr(sfbs), _ptr(sfao), _ptr(sfbo),
-                                      m, r if roomy else m, n, kn, ks, ko, _ptr(out), _stream(an))
+    status = lib().mg_mixed_gemm_ex(_ptr(an), _ptr(bn), _ptr(as_), _ptr(bs), _ptr(ao), _ptr(bo),
+                                    _ptr(sfan), _ptr(sfbn), _ptr(sfas), _ptr(sfbs), _ptr(sfao), _ptr(sfbo),
+                                    m, r if roomy else m, n, kn, ks, ko, MG_FLAG_W_TILED if w_tiled else 0,
+                                    _ptr(out), _stream(an))
     check(status, "mg_mixed_gemm")
     return out
 
 
-def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, workspace=None, out=None):
+def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, workspace=None, out=None, w_tiled=False):
     """Activation reorder-quantize + mixed GEMM on one stream; returns bf16 [M, N]."""
     _require(x, torch.bfloat16, "X")
     _require(reorder_index, torch.int16, "reorder_index")
@@ -186,11 +195,28 @@ def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, wor
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-    status = lib().mg_fused_linear(_ptr(x), _ptr(reorder_index), _ptr(bn), _ptr(bs), _ptr(bo),
-                                   _ptr(sfbn), _ptr(sfbs), _ptr(sfbo), m, n, kn, ks, ko,
-                                   _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
-    check(status, "mg_fused_linear")
+    status = lib().mg_fused_linear_ex(_ptr(x), _ptr(reorder_index), _ptr(bn), _ptr(bs), _ptr(bo),
+                                      _ptr(sfbn), _ptr(sfbs), _ptr(sfbo), m, n, kn, ks, ko,
+                                      MG_FLAG_W_TILED if w_tiled else 0,
+                                      _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
+    check(status, "mg_fused_linear_ex")
     return out
+
+
+def weights_tileable(n: int, kn: int, ks: int, ko: int) -> bool:
+    return bool(lib().mg_weights_tileable(n, kn, ks, ko))
+
+
+def tile_weights(wn, ws, wo):
+    """The three weight code tensors of reorder_quantize_w, rewritten into the tile-major order the
+    prefill kernel copies fastest (same shapes and sizes; pass w_tiled=True to matmul / fused_linear)."""
+    out = []
+    for t in (wn, ws, wo):
+        _require(t, torch.uint8, "weights")
+        dst = torch.empty_like(t)
+        check(lib().mg_tile_weights(_ptr(t), _ptr(dst), t.shape[0], t.shape[1] * 2, _stream(t)), "mg_tile_weights")
+        out.append(dst)
+    return tuple(out)
 
 
 def calibrate_reorder_index(x, out=None, workspace=None):

@@ -12,7 +12,8 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
 hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
-                             int a_rows, int N, int KN, int KS, int KO, void* d, hipStream_t stream);
+                             int a_rows, int N, int KN, int KS, int KO, unsigned flags, void* d, hipStream_t stream);
+hipError_t launch_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, hipStream_t stream);
 size_t calibrate_workspace_bytes(int K);
 hipError_t launch_calibrate(const void* x, int rows, int K, int16_t* idx, void* workspace, hipStream_t stream);
 }  // namespace mg
@@ -60,12 +61,14 @@ int mg_reorder_quantize_w(const void* w_bf16, const int16_t* idx, int N, int K, 
   return reorder_quantize<true>(w_bf16, idx, N, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream);
 }
 
-int mg_mixed_gemm_rows(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs, const uint8_t* ao,
-                       const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas,
-                       const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M, int a_rows, int N, int KN,
-                       int KS, int KO, void* d_bf16, void* stream) {
+int mg_mixed_gemm_ex(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs, const uint8_t* ao,
+                     const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas,
+                     const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M, int a_rows, int N, int KN,
+                     int KS, int KO, unsigned flags, void* d_bf16, void* stream) {
   if (int s = check_split(M, KN, KS, KO)) return s;
   if (N < 0 || a_rows < M) return MG_ERR_BAD_SHAPE;
+  if (flags & ~MG_FLAG_W_TILED) return MG_ERR_BAD_SHAPE;
+  if ((flags & MG_FLAG_W_TILED) && !mg_weights_tileable(N, KN, KS, KO)) return MG_ERR_UNSUPPORTED;
   if (M == 0 || N == 0) return MG_OK;
   if (!ptr_ok(d_bf16, true)) return MG_ERR_BAD_POINTER;
   if (!ptr_ok(an, KN > 0) || !ptr_ok(bn, KN > 0) || !ptr_ok(as_, KS > 0) || !ptr_ok(bs, KS > 0) ||
@@ -74,17 +77,28 @@ int mg_mixed_gemm_rows(const uint8_t* an, const uint8_t* bn, const uint8_t* as_,
   if ((KN > 0 && (!sfan || !sfbn)) || (KS > 0 && (!sfas || !sfbs)) || (KO > 0 && (!sfao || !sfbo)))
     return MG_ERR_BAD_POINTER;
   return (int)mg::launch_mixed_gemm(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, a_rows, N, KN, KS, KO,
-                                    d_bf16, static_cast<hipStream_t>(stream));
+                                    flags, d_bf16, static_cast<hipStream_t>(stream));
 }
 
 int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs, const uint8_t* ao,
                   const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
                   const uint8_t* sfao, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO, void* d_bf16,
                   void* stream) {
-  return mg_mixed_gemm_rows(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, M, N, KN, KS, KO, d_bf16, stream);
+  return mg_mixed_gemm_ex(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, M, N, KN, KS, KO, 0u, d_bf16, stream);
 }
 
 int mg_padded_rows(int M) { return M <= 0 ? 0 : (M + 255) / 256 * 256; }
+
+int mg_weights_tileable(int N, int KN, int KS, int KO) {
+  return N > 0 && N % 256 == 0 && KN >= 128 && KS >= 128 && KO >= 128 && (KN | KS | KO) % 128 == 0;
+}
+
+int mg_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, void* stream) {
+  if (N < 0 || kseg < 0 || N % 256 != 0 || kseg % 128 != 0) return MG_ERR_BAD_SHAPE;
+  if (N == 0 || kseg == 0) return MG_OK;
+  if (!ptr_ok(src, true) || !ptr_ok(dst, true) || src == dst) return MG_ERR_BAD_POINTER;
+  return (int)mg::launch_tile_weights(src, dst, N, kseg, static_cast<hipStream_t>(stream));
+}
 
 size_t mg_sf_bytes(int rows, int kseg, int operand) {
   if (rows < 0 || kseg < 0) return 0;
@@ -106,9 +120,9 @@ size_t mg_fused_workspace_bytes(int M, int KN, int KS, int KO) {
          align256(mg_sf_bytes(R, KO, MG_OPERAND_A));
 }
 
-int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
-                    const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO,
-                    void* d_bf16, void* workspace, size_t workspace_bytes, void* stream) {
+int mg_fused_linear_ex(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                       const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO,
+                       unsigned flags, void* d_bf16, void* workspace, size_t workspace_bytes, void* stream) {
   if (int s = check_split(M, KN, KS, KO)) return s;
   if (N < 0) return MG_ERR_BAD_SHAPE;
   if (M == 0 || N == 0) return MG_OK;
@@ -123,7 +137,14 @@ int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, c
   uint8_t* sfs = p; p += align256(mg_sf_bytes(R, KS, MG_OPERAND_A));
   uint8_t* sfo = p;
   if (int s = mg_reorder_quantize_x(x_bf16, idx, M, KN + KS + KO, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream)) return s;
-  return mg_mixed_gemm_rows(qn, bn, qs, bs, qo, bo, sfn, sfbn, sfs, sfbs, sfo, sfbo, M, R, N, KN, KS, KO, d_bf16, stream);
+  return mg_mixed_gemm_ex(qn, bn, qs, bs, qo, bo, sfn, sfbn, sfs, sfbs, sfo, sfbo, M, R, N, KN, KS, KO, flags, d_bf16, stream);
+}
+
+int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                    const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO,
+                    void* d_bf16, void* workspace, size_t workspace_bytes, void* stream) {
+  return mg_fused_linear_ex(x_bf16, idx, bn, bs, bo, sfbn, sfbs, sfbo, M, N, KN, KS, KO, 0u, d_bf16, workspace,
+                            workspace_bytes, stream);
 }
 
 size_t mg_calibrate_workspace_bytes(int K) { return K > 0 ? mg::calibrate_workspace_bytes(K) : 0; }

@@ -90,11 +90,11 @@ Tensor matmul(const Tensor& AN, const Tensor& BN, const Tensor& AS, const Tensor
                     capacity(SFAN) >= (int64_t)mg_sf_bytes(R, KN, MG_OPERAND_A) &&
                     capacity(SFAS) >= (int64_t)mg_sf_bytes(R, KS, MG_OPERAND_A) &&
                     capacity(SFAO) >= (int64_t)mg_sf_bytes(R, KO, MG_OPERAND_A);
-  const int status = mg_mixed_gemm_rows(AN.data_ptr<uint8_t>(), BN.data_ptr<uint8_t>(), AS.data_ptr<uint8_t>(),
+  const int status = mg_mixed_gemm_ex(AN.data_ptr<uint8_t>(), BN.data_ptr<uint8_t>(), AS.data_ptr<uint8_t>(),
                                         BS.data_ptr<uint8_t>(), AO.data_ptr<uint8_t>(), BO.data_ptr<uint8_t>(),
                                         SFAN.data_ptr<uint8_t>(), SFBN.data_ptr<uint8_t>(), SFAS.data_ptr<uint8_t>(),
                                         SFBS.data_ptr<uint8_t>(), SFAO.data_ptr<uint8_t>(), SFBO.data_ptr<uint8_t>(), M,
-                                        room ? R : M, N, KN, KS, KO, C.data_ptr<at::BFloat16>(), current_stream(AN));
+                                        room ? R : M, N, KN, KS, KO, 0u, C.data_ptr<at::BFloat16>(), current_stream(AN));
   finish(status, "GEMM");
   return C;
 }

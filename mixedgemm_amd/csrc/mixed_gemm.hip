@@ -161,12 +161,17 @@ __device__ __forceinline__ v4f decode_mfma(v8i wb, v8i xa, v4f acc, int sw, int 
 template <int G>
 __global__ void __launch_bounds__(256)
 mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, int M, int N, int steps_per_wave,
-                         uint16_t* __restrict__ d) {
+                         int w_tiled, uint16_t* __restrict__ d) {
   constexpr int S = G >= 8 ? 1 : 8 / G;   // K steps a wave keeps in flight at once
   __shared__ float partial[4][G][16 * 16];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, g = lane >> 4;
-  const int n = blockIdx.x * 16 + i;
+  // Row-major weights: the workgroup owns 16 consecutive features.  Tile-major weights: the 16 rows
+  // of one 1 KB copy block (block j = blockIdx.x % 16 of feature tile blockIdx.x / 16), i.e. features
+  // j + 16 * (2 * (t % 8) + t / 8) of the tile for t = 0..15, so that a weight load reads 1 KB of
+  // consecutive bytes.
+  const int tile_row0 = (blockIdx.x >> 4) * 256 + (blockIdx.x & 15);
+  const int n = w_tiled ? tile_row0 + 16 * (2 * (i & 7) + (i >> 3)) : blockIdx.x * 16 + i;
   const int m0 = m_base + blockIdx.y * (G * 16) + i;      // this lane's token in group 0
   const bool n_ok = n < N;
   const int nc = min(n, N - 1);   // clamped rows: every load is in bounds and unconditional
@@ -196,7 +201,11 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
       const int xbytes = seg == 0 ? 16 : (seg == 1 ? 24 : 32);   // activation bytes per 32-element block
       const int left = nblk - 4 * q;
       const int gc = min(g, left - 1);
-      wq[k] = *reinterpret_cast<const v4i*>(pb + (size_t)nc * nblk * 16 + q * 64 + gc * 16);
+      // tile-major weights: 16 KB per (256-feature tile, step), this workgroup's block in it, lane
+      // quad i, piece g; whole steps only
+      const size_t w_off = w_tiled ? ((((size_t)(blockIdx.x >> 4) * katoms + q) * 16 + (blockIdx.x & 15)) * 1024 + i * 64 + g * 16)
+                                   : ((size_t)nc * nblk * 16 + q * 64 + gc * 16);
+      wq[k] = *reinterpret_cast<const v4i*>(pb + w_off);
       sw[k] = psb[sf_offset(nc, 4 * q + gc, katoms)];
       // activations: two 16-byte pieces.  E2M1: block g (second piece unused);
       // E3M2: bytes [0,16) and [8,24) of block g; E4M3: K [16g,+16) and [64+16g,+16).
@@ -268,25 +277,34 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
     const int nn = blockIdx.x * 16 + 4 * g;
     const int m = m0 + gi * 16;
     if (m < M) {
-      uint16_t* dst = d + (size_t)m * N + nn;
+      if (w_tiled) {   // feature 4g + v of the workgroup is row tile_row0 + 16 * (2 * (t % 8) + t / 8), t = 4g + v
 #pragma unroll
-      for (int v = 0; v < 4; ++v)
-        if (nn + v < N) dst[v] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
+        for (int v = 0; v < 4; ++v) {
+          const int t = 4 * g + v;
+          d[(size_t)m * N + tile_row0 + 16 * (2 * (t & 7) + (t >> 3))] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
+        }
+      } else {
+        uint16_t* dst = d + (size_t)m * N + nn;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (nn + v < N) dst[v] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
+      }
     }
   }
 }
 
 hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int m_base, int M, int N,
-                         uint16_t* d, hipStream_t stream) {
+                         bool w_tiled, uint16_t* d, hipStream_t stream) {
   const int rows = M - m_base;
   const int steps_per_wave = (d4.steps + d6.steps + d8.steps + 3) / 4;
   const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
   const dim3 grid(ceil_div(N, 16), ceil_div(rows, 16 * g));
+  const int wt = w_tiled ? 1 : 0;
   switch (g) {
-    case 1: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<1>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, d); break;
-    case 2: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<2>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, d); break;
-    case 4: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<4>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, d); break;
-    default: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<8>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, d); break;
+    case 1: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<1>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d); break;
+    case 2: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<2>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d); break;
+    case 4: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<4>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d); break;
+    default: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<8>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d); break;
   }
   return hipGetLastError();
 }
@@ -581,7 +599,8 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO);
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
-                                 int M, int m_store, int N, int KN, int KS, int KO, void* d, hipStream_t stream);
+                                 int M, int m_store, int N, int KN, int KS, int KO, bool w_tiled, void* d,
+                                 hipStream_t stream);
 
 // Rough launch times in microseconds (measured on MI355X, K = 4096: a 128-wide stage takes ~1.05 us
 // with every CU busy and ~0.7 us when at most half of them are, plus ~8 us of fill and drain per
@@ -599,28 +618,31 @@ static double skinny_us(int rows, int N, int steps) {
 hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
-                             int a_rows, int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
+                             int a_rows, int N, int KN, int KS, int KO, unsigned flags, void* d, hipStream_t stream) {
   if (M == 0 || N == 0) return hipSuccess;
+  const bool w_tiled = (flags & 1u) != 0;   // MG_FLAG_W_TILED
+  // tile-major weights exist only for shapes the 256x256 kernel takes, in whole stages
+  if (w_tiled && (!mixed_gemm_256_supported(256, N, KN, KS, KO) || (KN | KS | KO) % 128 != 0)) return hipErrorInvalidValue;
   const int m_pad = (M + 255) / 256 * 256;
   const int steps = (KN + 127) / 128 + (KS + 127) / 128 + (KO + 127) / 128;
   // whole 256-row tiles, the last one possibly reading rows past M (readable up to a_rows) and
   // not writing them
   if ((M == m_pad || a_rows >= m_pad) && mixed_gemm_256_supported(m_pad, N, KN, KS, KO) &&
       (M >= 256 || pipelined_us(m_pad, N, steps) < skinny_us(M, N, steps)))
-    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_pad, M, N, KN, KS, KO, d,
-                                 stream);
+    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_pad, M, N, KN, KS, KO,
+                                 w_tiled, d, stream);
   const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
   const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
   const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};
-  if (M < 256 && KN + KS + KO > 0) return launch_skinny(d4, d6, d8, 0, M, N, static_cast<uint16_t*>(d), stream);
+  if (M < 256 && KN + KS + KO > 0) return launch_skinny(d4, d6, d8, 0, M, N, w_tiled, static_cast<uint16_t*>(d), stream);
   // ragged token count: whole 256-row tiles on the pipelined kernel (same pointers: rows are
   // independent and a scale atom never spans a 256-row boundary), the last rows on the skinny one
   const int m_main = M / 256 * 256;
   if (m_main < M && mixed_gemm_256_supported(m_main, N, KN, KS, KO)) {
     hipError_t e = launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_main, m_main, N, KN,
-                                         KS, KO, d, stream);
+                                         KS, KO, w_tiled, d, stream);
     if (e != hipSuccess) return e;
-    return launch_skinny(d4, d6, d8, m_main, M, N, static_cast<uint16_t*>(d), stream);
+    return launch_skinny(d4, d6, d8, m_main, M, N, w_tiled, static_cast<uint16_t*>(d), stream);
   }
   // the tiled kernel needs whole tiles and whole 128-wide K stages
   if (M % kTileM == 0 && N % kTileN == 0 && KN % kStageK == 0 && KS % kStageK == 0 && KO % kStageK == 0 &&

@@ -49,6 +49,7 @@ struct Plan {
   int st0, st1, st2;                  // whole 128-wide stages per segment
   int blk0, blk1, blk2;               // 32-element blocks per segment (row pitches and scale atoms; up to 3 more than 4 * st)
   int total;                          // stages over all segments
+  int w_tiled;                        // weights in tile-major order (see tile_weights_kernel): a copy reads 1 KB of consecutive bytes
 };
 
 __device__ __forceinline__ const uint8_t* uni(const uint8_t* p) {
@@ -116,9 +117,21 @@ __device__ __forceinline__ void copy16i(const uint8_t* base, unsigned voff, unsi
                : : "v"(voff), "s"(base), "s"(lds_sreg), "n"(OFF) : "memory", "m0", "scc");
 }
 
+// the same with an immediate byte offset on the global address as well.  The hardware adds the
+// instruction's immediate to the LDS address too, so M0 gets the LDS offset less the immediate.
+template <int OFF, int GOFF>
+__device__ __forceinline__ void copy16io(const uint8_t* base, unsigned voff, unsigned lds_sreg) {
+  static_assert(GOFF >= 0 && GOFF < 4096 && OFF >= GOFF, "global_load immediate offset");
+  base = uni(base);
+  lds_sreg = __builtin_amdgcn_readfirstlane(lds_sreg);
+  asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%4"
+               : : "v"(voff), "s"(base), "s"(lds_sreg), "n"(OFF - GOFF), "n"(GOFF) : "memory", "m0", "scc");
+}
+
 // Per-lane byte offsets of the copies, fixed for the whole kernel.
 struct LaneOffsets {
-  unsigned w0, w1, w2;      // 16 rows apart per lane quad, 64-byte rows of pitch ldb of segment 0 / 1 / 2 (also E2M1 tokens)
+  unsigned w0, w1, w2;      // weights: 16 rows apart per lane quad, 64-byte rows of pitch ldb of segment 0 / 1 / 2; tile-major: 16 * lane
+  unsigned x4;              // E2M1 tokens: the same pattern with the pitch of segment 0
   unsigned x8;              // E4M3 tokens: pitch lda of segment 2
   unsigned x6a, x6b, x6c;   // E3M2 tokens: piece (64k + lane) % 6 of row 8 * ((64k + lane) / 6), k = 0, 1, 2
   unsigned s0, s1, s2;      // scale atoms: lanes 0-31 the first 128 rows, 32-63 the next 128
@@ -127,9 +140,10 @@ struct LaneOffsets {
     // quad k of a copy holds tile row j + 16 * (2 * (k % 8) + k / 8): rows 32t + i and 32t + i + 16 of a
     // fragment end up 512 B apart in their block, which the LDS reads conflict-free (64 B apart they collide)
     const unsigned k = lane >> 2, pr = 2 * (k & 7) + (k >> 3), c = lane & 3;
-    w0 = 16 * pr * (p.blk0 * 16) + c * 16;
-    w1 = 16 * pr * (p.blk1 * 16) + c * 16;
-    w2 = 16 * pr * (p.blk2 * 16) + c * 16;
+    x4 = 16 * pr * (p.blk0 * 16) + c * 16;
+    w0 = p.w_tiled ? lane * 16 : x4;
+    w1 = p.w_tiled ? lane * 16 : 16 * pr * (p.blk1 * 16) + c * 16;
+    w2 = p.w_tiled ? lane * 16 : 16 * pr * (p.blk2 * 16) + c * 16;
     x8 = 16 * pr * (p.blk2 * 32) + c * 16;
     const unsigned lda6 = p.blk1 * 24, c0 = lane, c1 = 64 + lane, c2 = 128 + lane;
     x6a = 8 * (c0 / 6) * lda6 + (c0 % 6) * 16;
@@ -168,7 +182,14 @@ struct StageBases {
     const unsigned rb = sg == 0 ? 64 : (sg == 1 ? 96 : 128);
     ldb = blk * 16;
     lda = blk * (rb >> 2);
-    w = pb + (size_t)(c.n0 + c.wave * 4) * ldb + (size_t)ql * 64;
+    if (plan.w_tiled) {
+      // 16 KB per (feature tile, stage), 1 KB per copy block: the wave's 4 blocks are consecutive
+      const unsigned nstg = (unsigned)pick3(sg, (uint64_t)plan.st0, (uint64_t)plan.st1, (uint64_t)plan.st2);
+      w = pb + (((size_t)(c.n0 >> 8) * nstg + ql) * 16 + c.wave * 4) * 1024;
+      ldb = 1024;
+    } else {
+      w = pb + (size_t)(c.n0 + c.wave * 4) * ldb + (size_t)ql * 64;
+    }
     // first token row of the wave: E2M1 4*wave (+kx), E3M2 2*wave (+kx/3), E4M3 8*(wave%2) (+kx) in K half wave/2
     const unsigned xrow = sg == 0 ? c.wave * 4 : (sg == 1 ? c.wave * 2 : (c.wave & 1) * 8);
     x = pa + (size_t)(c.m0 + xrow) * lda + (size_t)ql * rb + (sg == 2 ? (c.wave >> 1) * 64 : 0);
@@ -197,7 +218,7 @@ struct GenericCopy {
     } else if constexpr (K < 12) {
       constexpr int kx = K - 4;
       if (b.seg == 0) {
-        if constexpr (kx < 4) copy16(b.x + (size_t)kx * b.lda, lo.w0, buf + kXOff + (wave * 4 + kx) * kBlk);
+        if constexpr (kx < 4) copy16(b.x + (size_t)kx * b.lda, lo.x4, buf + kXOff + (wave * 4 + kx) * kBlk);
       } else if (b.seg == 1) {
         if constexpr (kx < 6)
           copy16(b.x + (size_t)(kx / 3) * b.lda, kx % 3 == 0 ? lo.x6a : (kx % 3 == 1 ? lo.x6b : lo.x6c),
@@ -221,7 +242,9 @@ __device__ __forceinline__ void issue_range(const GenericCopy& cp, const LaneOff
 
 // Copies of stages inside one segment of format FMT: scalar bases advanced by one stage at a time,
 // per-lane offsets (one register per copy, the row step of the copy folded in) fixed.
-template <int FMT>
+// WT: weights in tile-major order -- one per-lane offset (16 * lane) and immediates for all four
+// weight copies; vw[] then holds the E2M1 token offsets only.
+template <int FMT, bool WT>
 struct LeanCopy {
   static constexpr int NX = Fmt<FMT>::x_copies;
   // token copies: E2M1 shares the weight offsets (same pitch); E3M2 keeps one offset per third of a
@@ -230,7 +253,7 @@ struct LeanCopy {
   const uint8_t *w, *x, *s;        // bases of the stage being copied
   unsigned lds_w, lds_x, lds_s;    // LDS offsets of the wave's first weight / token block and scale atom pair in buffer 0
   unsigned lda;
-  unsigned vw[4], vx[NV > 0 ? NV : 1], vs;
+  unsigned vw[4], vx[NV > 0 ? NV : 1], vs, vlin;
 
   __device__ __forceinline__ void init(const Plan& plan, int q, const LaneOffsets&, const Ctx& c) {
     const LaneOffsets lo(plan, c.lane);   // recomputed here rather than kept in registers across the K loop
@@ -241,8 +264,16 @@ struct LeanCopy {
     lda = __builtin_amdgcn_readfirstlane(b.lda);
     constexpr int sg = Fmt<FMT>::seg;
     const unsigned w_off = sg == 0 ? lo.w0 : (sg == 1 ? lo.w1 : lo.w2);
+    vlin = c.lane * 16;
+    if constexpr (WT) {
+      if constexpr (FMT == kFmtE2M1) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) vw[k] = w_off + k * b.ldb;
+        for (int k = 0; k < 4; ++k) vw[k] = lo.x4 + k * b.lda;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) vw[k] = w_off + k * b.ldb;   // E2M1 tokens use them too: same pattern, same pitch
+    }
     if constexpr (FMT == kFmtE3M2) {
       vx[0] = lo.x6a;
       vx[1] = lo.x6b;
@@ -260,7 +291,7 @@ struct LeanCopy {
   }
 
   __device__ __forceinline__ void advance() {
-    w += 64;
+    w += WT ? 16384 : 64;
     x += Fmt<FMT>::row_bytes;
     s += 512;
   }
@@ -271,7 +302,8 @@ struct LeanCopy {
   template <int K>
   __device__ __forceinline__ void issue(unsigned boff) const {
     if constexpr (K < 4) {
-      copy16i<K * kBlk>(w, vw[K], lds_w + boff);
+      if constexpr (WT) copy16io<K * kBlk, K * 1024>(w, vlin, lds_w + boff);
+      else copy16i<K * kBlk>(w, vw[K], lds_w + boff);
     } else if constexpr (K < 4 + NX) {
       constexpr int kx = K - 4;
       if constexpr (FMT == kFmtE2M1) copy16i<kx * kBlk>(x, vw[kx], lds_x + boff);
@@ -284,8 +316,8 @@ struct LeanCopy {
   }
 };
 
-template <>
-struct LeanCopy<kFmtNone> {
+template <bool WT>
+struct LeanCopy<kFmtNone, WT> {
   __device__ __forceinline__ void init(const Plan&, int, const LaneOffsets&, const Ctx&) {}
   __device__ __forceinline__ void advance() {}
   static constexpr int count() { return 0; }
@@ -439,9 +471,9 @@ constexpr int next_slot(int k) { return (k >= 4 + Fmt<FMT>::x_copies && k < 12) 
 // MFMAs stuck behind) and the copy slots [K0, K1) of one stage, one after every second MFMA.
 // LEAN: slots of `lc` (a stage of format CF, skipped when !on) into the buffer at byte offset boff;
 // otherwise slots of the run-time plan `gc`.
-template <int FMT, int H, bool LEAN, int CF, int M0, int K0, int K1, class Reader>
+template <int FMT, int H, bool LEAN, int CF, int M0, int K0, int K1, class Reader, bool WT>
 __device__ __forceinline__ void mfma_half(v16f (&acc)[4][4], const HalfFrags<FMT>& f, const Scales& sc, const Reader& rd,
-                                          const LeanCopy<CF>& lc, bool on, unsigned boff, const GenericCopy& gc,
+                                          const LeanCopy<CF, WT>& lc, bool on, unsigned boff, const GenericCopy& gc,
                                           const LaneOffsets& lo, int wave) {
   if constexpr (M0 < 16) {
     constexpr int tn = M0 / 4, tm = M0 % 4;
@@ -485,9 +517,9 @@ struct Ring {
 // (of stage q+3, format CE) from `lce` when early_on; MID says what happens to `lce` between the
 // halves: 1 = advance by one stage, 2 = set up for stage q+3 (first stage of its segment).
 // !LEAN: both from the run-time plan `gc`.  next_on: there is a stage q+1.
-template <int FMT, int FR, bool LEAN, int CL, int CE, int MID>
+template <int FMT, int FR, bool LEAN, int CL, int CE, int MID, bool WT>
 __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a, HalfFrags<FR>& a_next, Scales& sc,
-                                           const LeanCopy<CL>& lcl, bool late_on, LeanCopy<CE>& lce, bool early_on,
+                                           const LeanCopy<CL, WT>& lcl, bool late_on, LeanCopy<CE, WT>& lce, bool early_on,
                                            GenericCopy& gc, const LaneOffsets& lo, const Plan& plan, int q,
                                            bool next_on, const Ring& ring, const WeightPtrs& wp, const TokenPtrs<FMT>& xp,
                                            const TokenPtrs<FR>& xpn, const Ctx& c) {
@@ -501,7 +533,7 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
   if constexpr (LEAN) {
-    if (late_on) wait_copies_but_imm<LeanCopy<CL>::count()>();
+    if (late_on) wait_copies_but_imm<LeanCopy<CL, WT>::count()>();
     else wait_copies_but_imm<0>();
   } else {
     wait_copies_but(gc.count());
@@ -535,9 +567,9 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
 // `lcn`, which the next segment then continues to use as its `lc`.
 // !REGULAR: `gc` describes stage q0 + 2 (whose first copies are out) on entry and exit; the
 // stages that copy across a segment boundary take the run-time path.
-template <int FMT, int F1, int FR1, bool REGULAR>
+template <int FMT, int F1, int FR1, bool REGULAR, bool WT>
 __device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a, Scales& sc, HalfFrags<FR1>& a_next,
-                                            LeanCopy<FMT>& lc, LeanCopy<F1>& lcn, GenericCopy& gc, const LaneOffsets& lo,
+                                            LeanCopy<FMT, WT>& lc, LeanCopy<F1, WT>& lcn, GenericCopy& gc, const LaneOffsets& lo,
                                             const Plan& plan, int n, int n1, int q0, const WeightPtrs& wp,
                                             const uint8_t* lds, const Ctx& c) {
   const TokenPtrs<FMT> xp(lds, c);
@@ -656,8 +688,8 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
   }
 }
 
-// REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.
-template <bool REGULAR, bool REM>
+// REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
+template <bool REGULAR, bool REM, bool WT>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
@@ -673,6 +705,7 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* 
   plan.blk1 = __builtin_amdgcn_readfirstlane(plan_arg.blk1);
   plan.blk2 = __builtin_amdgcn_readfirstlane(plan_arg.blk2);
   plan.total = __builtin_amdgcn_readfirstlane(plan_arg.total);
+  plan.w_tiled = WT ? 1 : 0;
 
   const int tid = threadIdx.x;
   Ctx c;
@@ -742,10 +775,10 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* 
     wait_lds_reads();
     shift_scales(sc, sw, sx, c.lane);
   }
-  LeanCopy<kFmtE2M1> l4;
-  LeanCopy<kFmtE3M2> l6;
-  LeanCopy<kFmtE4M3> l8;
-  LeanCopy<kFmtNone> l0;
+  LeanCopy<kFmtE2M1, WT> l4;
+  LeanCopy<kFmtE3M2, WT> l6;
+  LeanCopy<kFmtE4M3, WT> l8;
+  LeanCopy<kFmtNone, WT> l0;
   if constexpr (REGULAR) l4.init(plan, 2, lo, c);
   run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
   run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
@@ -807,20 +840,25 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
-                                 int M, int m_store, int N, int KN, int KS, int KO, void* d, hipStream_t stream) {
+                                 int M, int m_store, int N, int KN, int KS, int KO, bool w_tiled, void* d,
+                                 hipStream_t stream) {
   // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
   const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
   const bool rem = (KN | KS | KO) % 128 != 0;
+  if (rem && w_tiled) return hipErrorInvalidValue;   // tile-major weights hold whole stages only
   typedef void (*kernel_t)(Plan, int, int, int, uint16_t*);
-  const kernel_t kernels[2][2] = {{mixed_gemm_256_kernel<false, false>, mixed_gemm_256_kernel<false, true>},
-                                  {mixed_gemm_256_kernel<true, false>, mixed_gemm_256_kernel<true, true>}};
-  const kernel_t kernel = kernels[regular][rem];
-  static bool configured[2][2] = {{false, false}, {false, false}};
-  if (!configured[regular][rem]) {
+  // [tiled][regular][rem]
+  const kernel_t kernels[2][2][2] = {
+      {{mixed_gemm_256_kernel<false, false, false>, mixed_gemm_256_kernel<false, true, false>},
+       {mixed_gemm_256_kernel<true, false, false>, mixed_gemm_256_kernel<true, true, false>}},
+      {{mixed_gemm_256_kernel<false, false, true>, nullptr}, {mixed_gemm_256_kernel<true, false, true>, nullptr}}};
+  const kernel_t kernel = kernels[w_tiled][regular][rem];
+  static bool configured[2][2][2] = {};
+  if (!configured[w_tiled][regular][rem]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        kBuffers * kStage);
     if (e != hipSuccess) return e;
-    configured[regular][rem] = true;
+    configured[w_tiled][regular][rem] = true;
   }
   Plan p;
   p.a0 = an; p.a1 = as_; p.a2 = ao;
@@ -830,9 +868,39 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.st0 = KN / 128; p.st1 = KS / 128; p.st2 = KO / 128;
   p.blk0 = KN / 32; p.blk1 = KS / 32; p.blk2 = KO / 32;
   p.total = p.st0 + p.st1 + p.st2;
+  p.w_tiled = w_tiled ? 1 : 0;
   const int tiles_n = N / kT, tiles_m = M / kT;
   hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store,
                      static_cast<uint16_t*>(d));
+  return hipGetLastError();
+}
+
+// Tile-major weight order of one segment (whole 128-wide stages, N a multiple of 256): per feature
+// tile of 256 rows and per stage one block of 16 KB, inside it the 16 copy blocks of 1 KB in the
+// order the kernel's LDS image wants them -- block j holds rows j + 16 * (2 * (k % 8) + k / 8) for
+// lane quad k = 0..15, 64 bytes (the stage's K range) each.  A copy instruction then reads 1 KB of
+// consecutive bytes (8 lines of 128 B) instead of 64 bytes from each of 16 rows (16 lines), and
+// the address unit, which limits the loop, has two thirds of the work.
+__global__ void __launch_bounds__(256) tile_weights_kernel(const v4u* __restrict__ src, v4u* __restrict__ dst, int N, int blk) {
+  const size_t total = (size_t)N * blk;   // 16-byte units
+  const int nst = blk >> 2;
+  for (size_t u = (size_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (size_t)gridDim.x * 256) {
+    const unsigned c = u & 3, k = (u >> 2) & 15, j = (u >> 6) & 15;
+    const size_t ts = u >> 10;   // tile_n * nst + stage
+    const unsigned ql = ts % nst;
+    const size_t tile_n = ts / nst;
+    const size_t row = tile_n * 256 + j + 16 * (2 * (k & 7) + (k >> 3));
+    dst[u] = src[row * blk + ql * 4 + c];
+  }
+}
+
+hipError_t launch_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, hipStream_t stream) {
+  if (N % 256 != 0 || kseg % 128 != 0) return hipErrorInvalidValue;
+  if (N == 0 || kseg == 0) return hipSuccess;
+  const size_t units = (size_t)N * (kseg / 32);
+  const int grid = (int)((units + 255) / 256 < 4096 ? (units + 255) / 256 : 4096);
+  hipLaunchKernelGGL(tile_weights_kernel, dim3(grid), dim3(256), 0, stream, reinterpret_cast<const v4u*>(src),
+                     reinterpret_cast<v4u*>(dst), N, kseg / 32);
   return hipGetLastError();
 }
 

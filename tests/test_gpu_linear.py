@@ -55,10 +55,12 @@ def test_pack_file_round_trip_through_the_gpu(linear, tmp_path):
     w = H.make_weights(n, k, 78)
     idx = H.absmax_sort_index(x)
     pw = linear.PackedWeights.from_float(w.to(DEV), idx.to(DEV), split)
+    assert not pw.tiled          # 48 features: not a multiple of 256
     torch.cuda.synchronize()
     path = str(tmp_path / "layer.mgw")
     pw.save(path)
     back = linear.PackedWeights.load(path, device=DEV)
+    assert not back.tiled
     for a, b in zip((*pw.tensors(), pw.reorder_index), (*back.tensors(), back.reorder_index)):
         assert torch.equal(a, b)
     y0 = linear.MixedLinear(pw)(x.to(DEV))
@@ -92,3 +94,28 @@ def test_operators_run_on_the_current_stream_without_synchronizing(linear):
     assert torch.equal(d0, d1) and torch.equal(d0, d2)
     for t0, t1 in zip(a[:3], a1[:3]):
         assert torch.equal(t0, t1)
+
+
+@pytest.mark.parametrize("m", [8, 300])
+def test_tiled_pack_round_trip_and_layer(linear, tmp_path, m):
+    """Default packing of a tileable layer is tile-major; the file keeps the layout and the layer gives
+    the row-major result bit for bit."""
+    n, k = 512, 4096
+    split = linear.default_split(k)
+    x = H.make_activations(m, k, 81)
+    w = H.make_weights(n, k, 82)
+    idx = H.absmax_sort_index(x)
+    tiled = linear.PackedWeights.from_float(w.to(DEV), idx.to(DEV), split)
+    plain = linear.PackedWeights.from_float(w.to(DEV), idx.to(DEV), split, tile=False)
+    assert tiled.tiled and not plain.tiled and not torch.equal(tiled.wn, plain.wn)
+    path = str(tmp_path / "tiled.mgw")
+    tiled.save(path)
+    assert linear.read_header(path)[0]["code_layout"] == "tile-major-256x128"
+    back = linear.PackedWeights.load(path, device=DEV)
+    assert back.tiled and torch.equal(back.wn, tiled.wn) and torch.equal(back.ws, tiled.ws)
+    y0 = linear.MixedLinear(plain)(x.to(DEV))
+    y1 = linear.MixedLinear(back)(x.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(y0, y1)
+    ref, slack = _oracle_linear(x, w, idx, split)
+    _close(y1, ref, slack)

@@ -352,3 +352,77 @@ def test_whole_path_matches_golden_vectors(abi, path):
     err = np.abs(d.float().cpu().numpy() - mo.bf16_rne(ref))
     # 1 bf16 ulp for the final rounding + 2^-20 of sum |a||b| for the order of the fp32 accumulation
     assert np.all(err <= H.bf16_ulp(ref) + g["d_abs_f32"] * 2.0 ** -20), f"max err {err.max()}"
+
+
+# ------------------------------------------------------------------ tile-major weights
+def _tile_reference(w: np.ndarray) -> np.ndarray:
+    """Tile-major order of one segment's weight codes [N, kseg/2] (N % 256 == 0, kseg % 128 == 0):
+    [feature tile][stage][block j][lane quad k][64 bytes], row = 256 * tile + j + 16 * (2 * (k % 8) + k // 8)."""
+    n, cols = w.shape
+    stages = cols // 64
+    v = w.reshape(n // 256, 256, stages, 64)
+    k = np.arange(16)
+    pr = 2 * (k % 8) + k // 8
+    rows = (np.arange(16)[:, None] + 16 * pr[None, :])            # [j, k]
+    out = v[:, rows, :, :]                                         # [tile, j, k, stage, 64]
+    return np.ascontiguousarray(out.transpose(0, 3, 1, 2, 4)).reshape(n, cols)
+
+
+@pytest.mark.parametrize("n,kseg", [(256, 128), (512, 384), (768, 2560)])
+def test_tile_weights_matches_the_layout_formula(abi, n, kseg):
+    rng = np.random.default_rng(n + kseg)
+    w = rng.integers(0, 256, (n, kseg // 2), dtype=np.uint8)
+    z = torch.zeros((n, 64), dtype=torch.uint8, device=DEV)
+    wd = torch.from_numpy(w).to(DEV)
+    t = abi.tile_weights(wd, wd[:, :64].contiguous(), wd[:, :64].contiguous())
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(t[0].cpu().numpy(), _tile_reference(w))
+    np.testing.assert_array_equal(t[1].cpu().numpy(), _tile_reference(w[:, :64]))
+    del z
+
+
+TILED_SHAPES = [
+    # M, N, KN, KS, KO: the 256x256 kernel (plain and with compiled-in segment-boundary copies), ragged
+    # token counts, and the skinny kernel with 1, 2, 4 and 8 token groups
+    (256, 256, 128, 128, 128), (512, 512, 256, 384, 128), (256, 768, 2560, 1408, 128), (512, 256, 384, 512, 256),
+    (300, 512, 2560, 1408, 128), (1000, 256, 384, 384, 384),
+    (8, 512, 2560, 1408, 128), (20, 256, 128, 256, 128), (50, 768, 384, 128, 128), (130, 256, 2560, 896, 128),
+]
+
+
+@pytest.mark.parametrize("m,n,kn,ks,ko", TILED_SHAPES)
+def test_tiled_weights_give_the_same_result_bit_for_bit(abi, m, n, kn, ks, ko):
+    """Tile-major weights change where a copy reads from, not what is multiplied or in which order."""
+    _say("tiled", m, n, kn, ks, ko)
+    k = kn + ks + ko
+    x = H.make_activations(m, k, 31 + m + n, n_out=max(1, k // 32))
+    w = H.make_weights(n, k, 33 + m + n)
+    idx = H.absmax_sort_index(x)
+    xd, wd, idd = x.to(DEV), w.to(DEV), idx.to(DEV)
+    assert abi.weights_tileable(n, kn, ks, ko)
+    bq = abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+    bt = abi.tile_weights(*bq[:3])
+    aq = abi.reorder_quantize_x(xd, idd, kn, ks, ko)
+    d0 = abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5])
+    d1 = abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], w_tiled=True)
+    d2 = abi.fused_linear(xd, idd, bt[0], bt[1], bt[2], bq[3], bq[4], bq[5], kn, ks, ko, w_tiled=True)
+    tight = [t.clone() for t in aq]    # exact-size activation buffers: whole tiles + skinny tail
+    d3 = abi.matmul(tight[0], bt[0], tight[1], bt[1], tight[2], bt[2], tight[3], bq[3], tight[4], bq[4], tight[5], bq[5],
+                    w_tiled=True)
+    torch.cuda.synchronize()
+    assert torch.equal(d0, d1) and torch.equal(d0, d2)
+    qx, qw = _oracle_operands(x, w, idx, kn, ks, ko)
+    _check_gemm(d1, qx, qw, "tiled")
+    _check_gemm(d3, qx, qw, "tiled, exact-size buffers")
+
+
+def test_tiled_flag_is_refused_for_shapes_that_cannot_be_tiled(abi):
+    from mixedgemm_amd.abi import MixedGemmError
+    assert not abi.weights_tileable(256, 448, 416, 224) and not abi.weights_tileable(200, 128, 128, 128)
+    m, n, kn, ks, ko = 16, 256, 448, 416, 224
+    x = H.make_activations(m, kn + ks + ko, 3).to(DEV)
+    idx = H.random_index(kn + ks + ko, 4).to(DEV)
+    aq = abi.reorder_quantize_x(x, idx, kn, ks, ko)
+    bq = abi.reorder_quantize_w(H.make_weights(n, kn + ks + ko, 5).to(DEV), idx, kn, ks, ko)
+    with pytest.raises(MixedGemmError):
+        abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], w_tiled=True)

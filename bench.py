@@ -204,6 +204,13 @@ def main():
                          "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("quant_c1"),
                          "algorithmic_bytes": qb},
         }
+        # ------------------------------------------------------------ c1 with an RMSNorm fused into the row pass
+        gamma1 = torch.ones(k1, dtype=torch.bfloat16, device=dev)
+        n_ms = graph_ms(lambda i: abi.rmsnorm_reorder_quantize_x(xs[i % nsets], gamma1, 1e-5, idx1, kn1, ks1, ko1,
+                                                                 out=outs[i % nsets]), iters)
+        extra["rmsnorm_reorder_quant_c1"] = {
+            "workload": "c1 with an RMSNorm in front, same pass (a separate RMSNorm kernel would read and write X once more)",
+            "value": round((qb + 2 * k1) / (n_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "avg_kernel_ms": round(n_ms, 5)}
         # ------------------------------------------------------------ calibration: column absmax + sort (reads X once)
         wsp = torch.empty(int(abi.lib().mg_calibrate_workspace_bytes(k1)), dtype=torch.uint8, device=dev)
         idx_out = torch.empty(k1, dtype=torch.int16, device=dev)

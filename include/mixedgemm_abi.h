@@ -61,6 +61,19 @@ int mg_reorder_quantize_w(const void* w_bf16, const int16_t* idx, int N, int K, 
                           uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream);
 
 /*
+ * mg_reorder_quantize_x with an RMSNorm in front, in the same pass over the rows (the layer that feeds
+ * a quantized linear in a transformer block; the reference leaves it to the caller and reads the
+ * normalised activations back from memory):
+ *   var = fl32( (sum of x^2 over the row, accumulated in fp64) / K ),  r = fl32( 1 / sqrt( fl32(var + eps) ) ),
+ *   y = bf16( gamma * bf16( x * r ) )   -- both products in fp32, gamma bf16 [K] --
+ * and y is what gets gathered and quantized.  eps >= 0.
+ */
+int mg_rmsnorm_reorder_quantize_x(const void* x_bf16, const void* gamma_bf16, float eps, const int16_t* idx,
+                                  int M, int K, int KN, int KS, int KO,
+                                  uint8_t* qn, uint8_t* qs, uint8_t* qo,
+                                  uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream);
+
+/*
  * Mixed block-scaled GEMM: D[M,N] = bf16( sum over the three K segments of
  * A_seg . B_seg^T ), fp32 accumulation across all segments, one bf16 rounding.
  * Replaces matmul_host (include/gemm.h:21-41, src/gemm.cu:22-47) and the three
@@ -119,6 +132,12 @@ int mg_fused_linear_ex(const void* x_bf16, const int16_t* idx,
                        const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo,
                        int M, int N, int KN, int KS, int KO, unsigned flags,
                        void* d_bf16, void* workspace, size_t workspace_bytes, void* stream);
+/* mg_fused_linear_ex with the RMSNorm of mg_rmsnorm_reorder_quantize_x in front (gamma_bf16 == NULL: none). */
+int mg_fused_norm_linear(const void* x_bf16, const void* gamma_bf16, float eps, const int16_t* idx,
+                         const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                         const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo,
+                         int M, int N, int KN, int KS, int KO, unsigned flags,
+                         void* d_bf16, void* workspace, size_t workspace_bytes, void* stream);
 size_t mg_fused_workspace_bytes(int M, int KN, int KS, int KO);
 
 /* Size in bytes of one segment's scale buffer (src/bindings.cpp:91-93, 210-212);

@@ -20,7 +20,7 @@ MG_FLAG_W_TILED = 1
 
 SYMBOLS = (
     "mg_reorder_quantize_x", "mg_reorder_quantize_w", "mg_mixed_gemm", "mg_mixed_gemm_ex", "mg_padded_rows", "mg_tile_weights",
-    "mg_weights_tileable", "mg_fused_linear_ex",
+    "mg_weights_tileable", "mg_fused_linear_ex", "mg_rmsnorm_reorder_quantize_x", "mg_fused_norm_linear",
     "mg_fused_linear",
     "mg_fused_workspace_bytes", "mg_sf_bytes", "mg_sf_offset", "mg_device_synchronize", "mg_status_string",
     "mg_measure_mfma_ceiling", "mg_calibrate_reorder_index", "mg_calibrate_workspace_bytes",
@@ -50,6 +50,11 @@ def lib() -> ctypes.CDLL:
         L.mg_mixed_gemm_ex.restype, L.mg_mixed_gemm_ex.argtypes = i, [p] * 12 + [i] * 6 + [u, p, p]
         L.mg_tile_weights.restype, L.mg_tile_weights.argtypes = i, [p, p, i, i, p]
         L.mg_weights_tileable.restype, L.mg_weights_tileable.argtypes = i, [i, i, i, i]
+        f = ctypes.c_float
+        L.mg_rmsnorm_reorder_quantize_x.restype = i
+        L.mg_rmsnorm_reorder_quantize_x.argtypes = [p, p, f, p, i, i, i, i, i, p, p, p, p, p, p, p]
+        L.mg_fused_norm_linear.restype = i
+        L.mg_fused_norm_linear.argtypes = [p, p, f, p] + [p] * 6 + [i] * 5 + [u, p, p, z, p]
         L.mg_fused_linear_ex.restype = i
         L.mg_fused_linear_ex.argtypes = [p] * 8 + [i] * 5 + [u, p, p, z, p]
         L.mg_padded_rows.restype, L.mg_padded_rows.argtypes = i, [i]
@@ -158,6 +163,24 @@ def reorder_quantize_x(x, reorder_index, kn, ks, ko, out=None):
     return _reorder_quantize("mg_reorder_quantize_x", MG_OPERAND_A, x, reorder_index, kn, ks, ko, out)
 
 
+def rmsnorm_reorder_quantize_x(x, norm_weight, eps, reorder_index, kn, ks, ko, out=None):
+    """reorder_quantize_x of RMSNorm(x) with bf16 weight norm_weight[K], in one pass over the rows
+    (the arithmetic is spelled out at mg_rmsnorm_reorder_quantize_x in the header)."""
+    _require(x, torch.bfloat16, "input")
+    _require(norm_weight, torch.bfloat16, "norm_weight")
+    _require(reorder_index, torch.int16, "reorder_index")
+    rows, k = x.shape
+    if reorder_index.numel() != k or norm_weight.numel() != k:
+        raise MixedGemmError(f"reorder_index / norm_weight must have {k} entries")
+    if out is None:
+        out = alloc_quant_outputs(rows, kn, ks, ko, MG_OPERAND_A, x.device)
+    qn, qs, qo, sfn, sfs, sfo = out
+    check(lib().mg_rmsnorm_reorder_quantize_x(_ptr(x), _ptr(norm_weight), float(eps), _ptr(reorder_index), rows, k, kn, ks,
+                                              ko, _ptr(qn), _ptr(qs), _ptr(qo), _ptr(sfn), _ptr(sfs), _ptr(sfo),
+                                              _stream(x)), "mg_rmsnorm_reorder_quantize_x")
+    return qn, qs, qo, sfn, sfs, sfo
+
+
 def reorder_quantize_w(w, reorder_index, kn, ks, ko, out=None):
     """(WN, WS, WO, SFWN, SFWS, SFWO); asynchronous on torch's current stream."""
     return _reorder_quantize("mg_reorder_quantize_w", MG_OPERAND_B, w, reorder_index, kn, ks, ko, out)
@@ -185,8 +208,10 @@ def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None
     return out
 
 
-def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, workspace=None, out=None, w_tiled=False):
-    """Activation reorder-quantize + mixed GEMM on one stream; returns bf16 [M, N]."""
+def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, workspace=None, out=None, w_tiled=False,
+                 norm_weight=None, eps=0.0):
+    """Activation reorder-quantize + mixed GEMM on one stream; returns bf16 [M, N].  With norm_weight
+    (bf16 [K]) the activations pass through an RMSNorm first, inside the quantizer's row pass."""
     _require(x, torch.bfloat16, "X")
     _require(reorder_index, torch.int16, "reorder_index")
     m, n = x.shape[0], bn.shape[0]
@@ -195,11 +220,15 @@ def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, wor
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-    status = lib().mg_fused_linear_ex(_ptr(x), _ptr(reorder_index), _ptr(bn), _ptr(bs), _ptr(bo),
-                                      _ptr(sfbn), _ptr(sfbs), _ptr(sfbo), m, n, kn, ks, ko,
-                                      MG_FLAG_W_TILED if w_tiled else 0,
-                                      _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
-    check(status, "mg_fused_linear_ex")
+    if norm_weight is not None:
+        _require(norm_weight, torch.bfloat16, "norm_weight")
+        if norm_weight.numel() != x.shape[1]:
+            raise MixedGemmError(f"norm_weight must have {x.shape[1]} entries")
+    status = lib().mg_fused_norm_linear(_ptr(x), _ptr(norm_weight), float(eps), _ptr(reorder_index), _ptr(bn), _ptr(bs),
+                                        _ptr(bo), _ptr(sfbn), _ptr(sfbs), _ptr(sfbo), m, n, kn, ks, ko,
+                                        MG_FLAG_W_TILED if w_tiled else 0,
+                                        _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
+    check(status, "mg_fused_norm_linear")
     return out
 
 

@@ -8,7 +8,8 @@
 namespace mg {
 template <bool IS_W>
 hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int K, int KN, int KS, int KO, uint8_t* qn,
-                                uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, hipStream_t stream);
+                                uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, const void* gamma,
+                                float eps, hipStream_t stream);
 hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
@@ -34,14 +35,15 @@ int check_split(int rows, int KN, int KS, int KO) {
 
 template <bool IS_W>
 int reorder_quantize(const void* x, const int16_t* idx, int rows, int K, int KN, int KS, int KO, uint8_t* qn,
-                     uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream) {
+                     uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream,
+                     const void* gamma = nullptr, float eps = 0.0f) {
   if (int s = check_split(rows, KN, KS, KO)) return s;
   if (K != KN + KS + KO) return MG_ERR_BAD_SHAPE;
   if (rows == 0 || K == 0) return MG_OK;
   if (!ptr_ok(x, true) || !ptr_ok(idx, true)) return MG_ERR_BAD_POINTER;
   if (!ptr_ok(qn, KN > 0) || !ptr_ok(qs, KS > 0) || !ptr_ok(qo, KO > 0)) return MG_ERR_BAD_POINTER;
   if ((KN > 0 && !sfn) || (KS > 0 && !sfs) || (KO > 0 && !sfo)) return MG_ERR_BAD_POINTER;
-  return (int)mg::launch_reorder_quant<IS_W>(x, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo,
+  return (int)mg::launch_reorder_quant<IS_W>(x, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, gamma, eps,
                                              static_cast<hipStream_t>(stream));
 }
 
@@ -54,6 +56,13 @@ extern "C" {
 int mg_reorder_quantize_x(const void* x_bf16, const int16_t* idx, int M, int K, int KN, int KS, int KO, uint8_t* qn,
                           uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream) {
   return reorder_quantize<false>(x_bf16, idx, M, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream);
+}
+
+int mg_rmsnorm_reorder_quantize_x(const void* x_bf16, const void* gamma_bf16, float eps, const int16_t* idx, int M, int K,
+                                  int KN, int KS, int KO, uint8_t* qn, uint8_t* qs, uint8_t* qo, uint8_t* sfn,
+                                  uint8_t* sfs, uint8_t* sfo, void* stream) {
+  if (!ptr_ok(gamma_bf16, true) || !(eps >= 0.0f)) return gamma_bf16 ? MG_ERR_BAD_SHAPE : MG_ERR_BAD_POINTER;
+  return reorder_quantize<false>(x_bf16, idx, M, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream, gamma_bf16, eps);
 }
 
 int mg_reorder_quantize_w(const void* w_bf16, const int16_t* idx, int N, int K, int KN, int KS, int KO, uint8_t* qn,
@@ -120,9 +129,11 @@ size_t mg_fused_workspace_bytes(int M, int KN, int KS, int KO) {
          align256(mg_sf_bytes(R, KO, MG_OPERAND_A));
 }
 
-int mg_fused_linear_ex(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
-                       const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO,
-                       unsigned flags, void* d_bf16, void* workspace, size_t workspace_bytes, void* stream) {
+int mg_fused_norm_linear(const void* x_bf16, const void* gamma_bf16, float eps, const int16_t* idx, const uint8_t* bn,
+                         const uint8_t* bs, const uint8_t* bo, const uint8_t* sfbn, const uint8_t* sfbs,
+                         const uint8_t* sfbo, int M, int N, int KN, int KS, int KO, unsigned flags, void* d_bf16,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+  if (gamma_bf16 != nullptr && !(eps >= 0.0f)) return MG_ERR_BAD_SHAPE;
   if (int s = check_split(M, KN, KS, KO)) return s;
   if (N < 0) return MG_ERR_BAD_SHAPE;
   if (M == 0 || N == 0) return MG_OK;
@@ -136,8 +147,16 @@ int mg_fused_linear_ex(const void* x_bf16, const int16_t* idx, const uint8_t* bn
   uint8_t* sfn = p; p += align256(mg_sf_bytes(R, KN, MG_OPERAND_A));
   uint8_t* sfs = p; p += align256(mg_sf_bytes(R, KS, MG_OPERAND_A));
   uint8_t* sfo = p;
-  if (int s = mg_reorder_quantize_x(x_bf16, idx, M, KN + KS + KO, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream)) return s;
+  if (int s = reorder_quantize<false>(x_bf16, idx, M, KN + KS + KO, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream, gamma_bf16, eps))
+    return s;
   return mg_mixed_gemm_ex(qn, bn, qs, bs, qo, bo, sfn, sfbn, sfs, sfbs, sfo, sfbo, M, R, N, KN, KS, KO, flags, d_bf16, stream);
+}
+
+int mg_fused_linear_ex(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                       const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo, int M, int N, int KN, int KS, int KO,
+                       unsigned flags, void* d_bf16, void* workspace, size_t workspace_bytes, void* stream) {
+  return mg_fused_norm_linear(x_bf16, nullptr, 0.0f, idx, bn, bs, bo, sfbn, sfbs, sfbo, M, N, KN, KS, KO, flags, d_bf16,
+                              workspace, workspace_bytes, stream);
 }
 
 int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,

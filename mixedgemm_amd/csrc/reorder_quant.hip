@@ -105,12 +105,22 @@ __device__ __forceinline__ void quantize_store(const float (&f)[32], int fmt, ui
 // issued before the current group is gathered and quantized, and the LDS tile is double buffered
 // (buf_stride bytes apart; 0 when every workgroup has a single group), so loads, arithmetic and
 // stores of different groups overlap inside the workgroup and one barrier per group suffices.
-template <int R, bool IS_W, int MAXT>
+//
+// NORM: an RMSNorm (weight gamma, bf16 in and out, the arithmetic of the usual fp32 implementation)
+// is applied to each row before the gather:
+//   var = fl32( (sum over the row of x^2, accumulated in fp64) / K )
+//   r   = fl32( 1 / sqrt( fl32(var + eps) ) )      (division and square root in fp64)
+//   y   = bf16( gamma * bf16( x * r ) )            (both products in fp32)
+// The fp64 sum makes the result independent of the order in which the lanes add their parts
+// (up to the last bit of a double, which the rounding to fp32 all but never sees).
+template <int R, bool IS_W, int MAXT, bool NORM>
 __global__ void __launch_bounds__(MAXT)
 reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__ idx, int rows, int K, int KN, int KS,
                      int KO, uint8_t* __restrict__ qn, uint8_t* __restrict__ qs, uint8_t* __restrict__ qo,
-                     uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo, int buf_stride) {
+                     uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo, int buf_stride,
+                     const uint16_t* __restrict__ gamma, float eps) {
   extern __shared__ __align__(16) uint8_t lds_all[];
+  __shared__ double row_sums[R][MAXT / 64];
   const int tid = threadIdx.x;
   const int nthr = blockDim.x;
   const int ngroups = (rows + R - 1) / R;
@@ -159,10 +169,57 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
   int group = blockIdx.x;
   if (group >= ngroups) return;
   issue_loads(group);
+  v4u gv[4];   // the RMSNorm weights of this lane's chunks (the same for every row)
+  if constexpr (NORM) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it)
+      gv[it] = *reinterpret_cast<const v4u*>(gamma + (size_t)min(tid + it * nthr, nchunks - 1) * 8);
+  }
   int parity = 0;
   for (; group < ngroups; group += gridDim.x, parity ^= 1) {
     uint8_t* lds = lds_all + parity * buf_stride;
     const int row0 = group * R;
+    if constexpr (NORM) {
+      double ss[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        ss[r] = 0.0;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          if (tid + it * nthr < nchunks) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const unsigned d = a[it][r][e];
+              const double lo = (double)__uint_as_float(d << 16), hi = (double)__uint_as_float(d & 0xffff0000u);
+              ss[r] = __builtin_fma(lo, lo, ss[r]);
+              ss[r] = __builtin_fma(hi, hi, ss[r]);
+            }
+          }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) ss[r] += __shfl_xor(ss[r], off, 64);
+        if ((tid & 63) == 0) row_sums[r][tid >> 6] = ss[r];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        double tot = 0.0;
+        for (int w = 0; w < (nthr >> 6); ++w) tot += row_sums[r][w];
+        const float var = (float)(tot / (double)K);
+        const float rn = (float)(1.0 / __builtin_sqrt((double)(var + eps)));
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const unsigned d = a[it][r][e], g = gv[it][e];
+            const float h0 = (float)(__bf16)(__uint_as_float(d << 16) * rn);
+            const float h1 = (float)(__bf16)(__uint_as_float(d & 0xffff0000u) * rn);
+            const v2bf y = {(__bf16)(__uint_as_float(g << 16) * h0), (__bf16)(__uint_as_float(g & 0xffff0000u) * h1)};
+            a[it][r][e] = __builtin_bit_cast(unsigned, y);
+          }
+        }
+      }
+    }
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
       const int c = tid + it * nthr;
@@ -238,11 +295,14 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
 
 }  // namespace
 
+// gamma != nullptr: RMSNorm with that weight and eps before the gather (activations only)
 template <bool IS_W>
 hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int K, int KN, int KS, int KO, uint8_t* qn,
                                 uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo,
-                                hipStream_t stream) {
+                                const void* gamma, float eps, hipStream_t stream) {
   if (rows == 0 || K == 0) return hipSuccess;
+  if (gamma != nullptr && IS_W) return hipErrorInvalidValue;
+  const uint16_t* gm = static_cast<const uint16_t*>(gamma);
   const int threads = ((K >> 5) + 63) & ~63;
   const uint16_t* xb = static_cast<const uint16_t*>(x);
   // R rows interleaved in LDS.  More row groups than `resident` workgroups: each workgroup
@@ -259,25 +319,33 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
     const bool stream_groups = ngroups > resident && 2 * tile <= 160 * 1024;
     const int grid = stream_groups ? resident : ngroups;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), (size_t)(stream_groups ? 2 * tile : tile), stream, xb, idx, rows, K,
-                       KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream_groups ? tile : 0);
+                       KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream_groups ? tile : 0, gm, eps);
   };
 #ifndef MG_QUANT_R_SMALLK
 #define MG_QUANT_R_SMALLK 1
 #endif
+  constexpr int R = MG_QUANT_R_SMALLK;
+  if constexpr (!IS_W) {
+    if (gamma != nullptr) {
+      if (K <= 8192) launch(reorder_quant_kernel<R, false, 256, true>, R);
+      else if (K <= 16384) launch(reorder_quant_kernel<2, false, 512, true>, 2);
+      else launch(reorder_quant_kernel<1, false, 1024, true>, 1);
+      return hipGetLastError();
+    }
+  }
   if (K <= 8192) {
-    constexpr int R = MG_QUANT_R_SMALLK;
-    launch(reorder_quant_kernel<R, IS_W, 256>, R);
+    launch(reorder_quant_kernel<R, IS_W, 256, false>, R);
   } else if (K <= 16384) {
-    launch(reorder_quant_kernel<2, IS_W, 512>, 2);
+    launch(reorder_quant_kernel<2, IS_W, 512, false>, 2);
   } else {
-    launch(reorder_quant_kernel<1, IS_W, 1024>, 1);
+    launch(reorder_quant_kernel<1, IS_W, 1024, false>, 1);
   }
   return hipGetLastError();
 }
 
 template hipError_t launch_reorder_quant<false>(const void*, const int16_t*, int, int, int, int, int, uint8_t*, uint8_t*,
-                                                uint8_t*, uint8_t*, uint8_t*, uint8_t*, hipStream_t);
+                                                uint8_t*, uint8_t*, uint8_t*, uint8_t*, const void*, float, hipStream_t);
 template hipError_t launch_reorder_quant<true>(const void*, const int16_t*, int, int, int, int, int, uint8_t*, uint8_t*,
-                                               uint8_t*, uint8_t*, uint8_t*, uint8_t*, hipStream_t);
+                                               uint8_t*, uint8_t*, uint8_t*, uint8_t*, const void*, float, hipStream_t);
 
 }  // namespace mg

@@ -240,6 +240,20 @@ def _(X, reorder_index, BN, BS, BO, SFBN, SFBS, SFBO, KN, KS, KO, w_tiled=False)
     return torch.empty((X.shape[0], n), dtype=torch.bfloat16, device=X.device)
 
 
+@torch.library.custom_op("mixedgemm_amd::fused_norm_linear", mutates_args=())
+def fused_norm_linear_op(X: torch.Tensor, norm_weight: torch.Tensor, eps: float, reorder_index: torch.Tensor,
+                         BN: torch.Tensor, BS: torch.Tensor, BO: torch.Tensor, SFBN: torch.Tensor, SFBS: torch.Tensor,
+                         SFBO: torch.Tensor, KN: int, KS: int, KO: int, w_tiled: bool = False) -> torch.Tensor:
+    return abi.fused_linear(X, reorder_index, BN, BS, BO, SFBN, SFBS, SFBO, KN, KS, KO, w_tiled=w_tiled,
+                            norm_weight=norm_weight, eps=eps)
+
+
+@fused_norm_linear_op.register_fake
+def _(X, norm_weight, eps, reorder_index, BN, BS, BO, SFBN, SFBS, SFBO, KN, KS, KO, w_tiled=False):
+    n = BN.shape[0] if KN else (BS.shape[0] if KS else BO.shape[0])
+    return torch.empty((X.shape[0], n), dtype=torch.bfloat16, device=X.device)
+
+
 @torch.library.custom_op("mixedgemm_amd::calibrate_reorder_index", mutates_args=())
 def calibrate_reorder_index_op(X: torch.Tensor) -> torch.Tensor:
     return abi.calibrate_reorder_index(X)
@@ -253,10 +267,14 @@ def _(X):
 # ------------------------------------------------------------------ the layer
 class MixedLinear(torch.nn.Module):
     """y = quantize(x[..., reorder_index]) @ Wq^T (+ bias): the reference's three calls
-    (main.py:35-37) with the weights quantized once.  Inference only."""
+    (main.py:35-37) with the weights quantized once.  Inference only.  With norm_weight (bf16 [K]) the
+    input first passes through an RMSNorm, computed inside the quantizer's pass over the rows; the
+    reorder index must then have been calibrated on normalised activations."""
 
-    def __init__(self, packed: PackedWeights, bias: torch.Tensor | None = None):
+    def __init__(self, packed: PackedWeights, bias: torch.Tensor | None = None,
+                 norm_weight: torch.Tensor | None = None, eps: float = 1e-5):
         super().__init__()
+        self.eps = float(eps)
         packed.validate()
         self.split = packed.split
         self.tiled = packed.tiled
@@ -264,6 +282,7 @@ class MixedLinear(torch.nn.Module):
         for name in _SECTIONS:
             self.register_buffer(name, getattr(packed, name))
         self.register_buffer("bias", bias)
+        self.register_buffer("norm_weight", norm_weight)
 
     @classmethod
     def from_float(cls, weight: torch.Tensor, calibration_x: torch.Tensor | None = None,
@@ -286,8 +305,13 @@ class MixedLinear(torch.nn.Module):
         x2 = x.reshape(-1, self.in_features)
         if x2.dtype != torch.bfloat16:
             x2 = x2.to(torch.bfloat16)
-        y = torch.ops.mixedgemm_amd.fused_linear(x2.contiguous(), self.reorder_index, self.wn, self.ws, self.wo,
-                                                 self.sfwn, self.sfws, self.sfwo, *self.split, self.tiled)
+        if self.norm_weight is not None:
+            y = torch.ops.mixedgemm_amd.fused_norm_linear(x2.contiguous(), self.norm_weight, self.eps, self.reorder_index,
+                                                          self.wn, self.ws, self.wo, self.sfwn, self.sfws, self.sfwo,
+                                                          *self.split, self.tiled)
+        else:
+            y = torch.ops.mixedgemm_amd.fused_linear(x2.contiguous(), self.reorder_index, self.wn, self.ws, self.wo,
+                                                     self.sfwn, self.sfws, self.sfwo, *self.split, self.tiled)
         if self.bias is not None:
             y = y + self.bias
         return y.reshape(*lead, self.out_features)

@@ -346,3 +346,23 @@ def calibrate_reorder_index(x_bits):
     orders like |x|, so no float conversion is needed."""
     mag = (np.asarray(x_bits, dtype=np.uint16) & 0x7FFF).max(axis=0).astype(np.uint32)
     return np.argsort(mag, kind="stable").astype(np.int16)
+
+
+def rmsnorm_bf16(x_bits, gamma_bits, eps):
+    """RMSNorm of bf16 rows x[M, K] with bf16 weight gamma[K], as bf16 bit patterns -- the
+    arithmetic the usual fp32 implementation spells out (to fp32, mean of squares, rsqrt, back to
+    bf16, times the weight), with the reduction and the reciprocal square root pinned so that the
+    result does not depend on who computes it:
+        var = fl32( (sum of x^2 in float64) / K );  r = fl32( 1 / sqrt( fl32(var + eps) ) )  in float64;
+        y   = bf16( gamma * bf16( x * r ) ), both products in float32.
+    The reference has no normalisation layer: this is the layer in front of a quantized linear."""
+    x = (np.asarray(x_bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+    g = (np.asarray(gamma_bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+    k = x.shape[1]
+    ss = (x.astype(np.float64) ** 2).sum(axis=1)
+    var = (ss / np.float64(k)).astype(np.float32)
+    t = (var + np.float32(eps)).astype(np.float32)
+    r = (1.0 / np.sqrt(t.astype(np.float64))).astype(np.float32)
+    h = bf16_rne((x * r[:, None]).astype(np.float32))
+    y = bf16_rne((g[None, :] * h).astype(np.float32))
+    return (y.view(np.uint32) >> 16).astype(np.uint16)

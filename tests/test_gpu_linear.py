@@ -119,3 +119,20 @@ def test_tiled_pack_round_trip_and_layer(linear, tmp_path, m):
     assert torch.equal(y0, y1)
     ref, slack = _oracle_linear(x, w, idx, split)
     _close(y1, ref, slack)
+
+
+def test_layer_with_fused_rmsnorm(linear):
+    m, n, k, eps = 70, 256, 4096, 1e-5
+    split = linear.default_split(k)
+    x = H.make_activations(m, k, 91)
+    w = H.make_weights(n, k, 92)
+    g = torch.Generator().manual_seed(93)
+    gamma = (torch.randn(k, generator=g) * 0.3 + 1.0).to(torch.bfloat16)
+    y = torch.from_numpy(mo.rmsnorm_bf16(H.bf16_bits(x), H.bf16_bits(gamma), eps).view(np.int16)).view(torch.bfloat16)
+    idx = H.absmax_sort_index(y)
+    pw = linear.PackedWeights.from_float(w.to(DEV), idx.to(DEV), split)
+    layer = linear.MixedLinear(pw, norm_weight=gamma.to(DEV), eps=eps)
+    out = layer(x.to(DEV))
+    torch.cuda.synchronize()
+    ref, slack = _oracle_linear(y, w, idx, split)
+    _close(out, ref, slack)

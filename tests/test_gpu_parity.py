@@ -426,3 +426,43 @@ def test_tiled_flag_is_refused_for_shapes_that_cannot_be_tiled(abi):
     bq = abi.reorder_quantize_w(H.make_weights(n, kn + ks + ko, 5).to(DEV), idx, kn, ks, ko)
     with pytest.raises(MixedGemmError):
         abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], w_tiled=True)
+
+
+# ------------------------------------------------------------------ RMSNorm fused into the quantizer
+@pytest.mark.parametrize("rows,kn,ks,ko,eps", [
+    (7, 2560, 1408, 128, 1e-5), (130, 2560, 896, 128, 1e-6), (5, 128, 64, 64, 0.0),
+    (9, 8960, 4928, 448, 1e-5),      # two rows per pass
+    (3, 11776, 6560, 608, 1e-5),     # K = 18944: 1024-lane workgroups
+    (1030, 256, 128, 128, 1e-5),     # more row groups than resident workgroups: streamed
+])
+def test_rmsnorm_reorder_quantize_matches_oracle(abi, rows, kn, ks, ko, eps):
+    k = kn + ks + ko
+    _say("norm quant", rows, kn, ks, ko)
+    x = H.make_activations(rows, k, 300 + rows, n_out=max(1, k // 32))
+    g = torch.Generator().manual_seed(rows)
+    gamma = (torch.randn(k, generator=g) * 0.3 + 1.0).to(torch.bfloat16)
+    idx = H.random_index(k, 301 + rows)
+    got = abi.rmsnorm_reorder_quantize_x(x.to(DEV), gamma.to(DEV), eps, idx.to(DEV), kn, ks, ko)
+    torch.cuda.synchronize()
+    y_bits = mo.rmsnorm_bf16(H.bf16_bits(x), H.bf16_bits(gamma), eps)
+    want = sc.quantize_x(y_bits, idx.numpy(), kn, ks, ko)
+    H.assert_quant_equal(got, want, rows, (kn, ks, ko), what=f"norm x {rows}x{k}")
+
+
+def test_fused_norm_linear_equals_norm_then_linear(abi):
+    m, n, kn, ks, ko, eps = 300, 512, 2560, 1408, 128, 1e-5
+    k = kn + ks + ko
+    x = H.make_activations(m, k, 61)
+    w = H.make_weights(n, k, 62)
+    g = torch.Generator().manual_seed(63)
+    gamma = (torch.randn(k, generator=g) * 0.3 + 1.0).to(torch.bfloat16)
+    y = torch.from_numpy(mo.rmsnorm_bf16(H.bf16_bits(x), H.bf16_bits(gamma), eps).view(np.int16)).view(torch.bfloat16)
+    idx = H.absmax_sort_index(y)
+    xd, wd, idd = x.to(DEV), w.to(DEV), idx.to(DEV)
+    bq = abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+    d1 = abi.fused_linear(xd, idd, *bq, kn, ks, ko, norm_weight=gamma.to(DEV), eps=eps)
+    d2 = abi.fused_linear(y.to(DEV), idd, *bq, kn, ks, ko)
+    torch.cuda.synchronize()
+    assert torch.equal(d1, d2)
+    qx, qw = _oracle_operands(y, w, idx, kn, ks, ko)
+    _check_gemm(d1, qx, qw, "fused norm linear")

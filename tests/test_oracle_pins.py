@@ -359,3 +359,52 @@ def test_calibrate_index_is_a_permutation_sorted_by_absmax():
     assert sorted(idx.tolist()) == list(range(4096))
     am = x.float().abs().max(dim=0).values.numpy()
     assert np.all(np.diff(am[idx]) >= 0)
+
+
+# ------------------------------------------------------------------ RMSNorm in front of the quantizer
+def _bits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _from_bits(b):
+    return torch.from_numpy(np.ascontiguousarray(b).view(np.int16)).view(torch.bfloat16)
+
+
+def test_rmsnorm_closed_forms():
+    """Cases whose answer is known without the formula: a constant row normalises to +-1, so y is the
+    weight itself (a sum in place of the mean, a missing square root or a dropped weight all fail this);
+    scaling a row by a power of two changes nothing when eps = 0; a zero row stays zero with eps > 0."""
+    g = torch.Generator().manual_seed(3)
+    k = 256
+    gamma = (torch.randn(k, generator=g) * 0.5 + 1.0).to(torch.bfloat16)
+    x = torch.full((3, k), 1.5, dtype=torch.bfloat16)
+    x[1] = -0.375
+    x[2, ::2] = -1.5                                   # |x| constant, signs alternate
+    y = _from_bits(mo.rmsnorm_bf16(_bits(x), _bits(gamma), 0.0)).float()
+    np.testing.assert_array_equal(y[0].numpy(), gamma.float().numpy())
+    np.testing.assert_array_equal(y[1].numpy(), -gamma.float().numpy())
+    sign = torch.ones(k); sign[::2] = -1
+    np.testing.assert_array_equal(y[2].numpy(), (gamma.float() * sign).numpy())
+    xr = torch.randn(4, k, generator=g).to(torch.bfloat16)
+    a = mo.rmsnorm_bf16(_bits(xr), _bits(gamma), 0.0)
+    b = mo.rmsnorm_bf16(_bits((xr.float() * 64.0).to(torch.bfloat16)), _bits(gamma), 0.0)
+    np.testing.assert_array_equal(a, b)
+    z = mo.rmsnorm_bf16(_bits(torch.zeros(1, k, dtype=torch.bfloat16)), _bits(gamma), 1e-6)
+    assert not (z & 0x7FFF).any()
+
+
+def test_rmsnorm_agrees_with_the_usual_fp32_implementation():
+    """torch, written the way transformer code writes it.  Its float32 mean and rsqrt may differ from the
+    pinned float64 ones in the last bit, which can move a bf16 rounding: at most a few values per
+    thousand may differ, each by one bf16 step."""
+    g = torch.Generator().manual_seed(4)
+    m, k, eps = 16, 4096, 1e-5
+    x = (torch.randn(m, k, generator=g) * 3.0).to(torch.bfloat16)
+    gamma = (torch.randn(k, generator=g) * 0.2 + 1.0).to(torch.bfloat16)
+    h = x.float()
+    var = h.pow(2).mean(-1, keepdim=True)
+    ref = gamma * (h * torch.rsqrt(var + eps)).to(torch.bfloat16)
+    got = _from_bits(mo.rmsnorm_bf16(_bits(x), _bits(gamma), eps))
+    diff = (got.view(torch.int16).int() - ref.view(torch.int16).int()).abs()
+    assert int(diff.max()) <= 1
+    assert float((diff != 0).float().mean()) < 5e-3

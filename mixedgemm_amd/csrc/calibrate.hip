@@ -134,13 +134,8 @@ hipError_t launch_calibrate(const void* x, int rows, int K, int16_t* idx, void* 
   hipLaunchKernelGGL(channel_keys_kernel, dim3(ceil_div(K, 64)), dim3(256), 0, stream, partial, nstrips, K, keys);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  static bool configured = false;
-  if (!configured) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(rank_channels_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (32768 + kRankWaves * 64) * sizeof(unsigned));
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  e = allow_dynamic_lds(reinterpret_cast<const void*>(rank_channels_kernel), (32768 + kRankWaves * 64) * (int)sizeof(unsigned));
+  if (e != hipSuccess) return e;
   hipLaunchKernelGGL(rank_channels_kernel, dim3(ceil_div(K, 64)), dim3(kRankWaves * 64),
                      (size_t)(K + kRankWaves * 64) * sizeof(unsigned), stream, keys, K, idx);
   return hipGetLastError();

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 namespace mg {
 
 constexpr int kGroup = 32;  // elements per shared scale (src/reorder.cu:78-79 of the reference)
@@ -32,5 +34,30 @@ __host__ __device__ inline size_t sf_offset(int r, int kb, int katoms) {
 }
 
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Raises a kernel's dynamic-LDS limit to `bytes`, once per kernel and device (the attribute is kept
+// per device); safe to call from several host threads.
+inline hipError_t allow_dynamic_lds(const void* kernel, int bytes) {
+  struct Entry { const void* kernel; uint64_t devices; };
+  static std::mutex mu;
+  static Entry table[32] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  std::lock_guard<std::mutex> lock(mu);
+  Entry* slot = nullptr;
+  for (Entry& t : table) {
+    if (t.kernel == kernel) { slot = &t; break; }
+    if (t.kernel == nullptr && slot == nullptr) slot = &t;
+  }
+  if (slot != nullptr && slot->kernel == kernel && (slot->devices & bit)) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && slot != nullptr) {
+    slot->kernel = kernel;
+    slot->devices |= bit;
+  }
+  return e;
+}
 
 }  // namespace mg

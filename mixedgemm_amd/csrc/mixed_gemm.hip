@@ -647,13 +647,8 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
   // the tiled kernel needs whole tiles and whole 128-wide K stages
   if (M % kTileM == 0 && N % kTileN == 0 && KN % kStageK == 0 && KS % kStageK == 0 && KO % kStageK == 0 &&
       KN + KS + KO > 0) {
-    static bool configured = false;
-    if (!configured) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mixed_gemm_tiled_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kStageBytes);
-      if (e != hipSuccess) return e;
-      configured = true;
-    }
+    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(mixed_gemm_tiled_kernel), 2 * kStageBytes);
+    if (e != hipSuccess) return e;
     const Seg s4 = {an, bn, sfan, sfbn, KN / kStageK};
     const Seg s6 = {as_, bs, sfas, sfbs, KS / kStageK};
     const Seg s8 = {ao, bo, sfao, sfbo, KO / kStageK};

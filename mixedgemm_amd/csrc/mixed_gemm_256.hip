@@ -853,13 +853,7 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
        {mixed_gemm_256_kernel<true, false, false>, mixed_gemm_256_kernel<true, true, false>}},
       {{mixed_gemm_256_kernel<false, false, true>, nullptr}, {mixed_gemm_256_kernel<true, false, true>, nullptr}}};
   const kernel_t kernel = kernels[w_tiled][regular][rem];
-  static bool configured[2][2][2] = {};
-  if (!configured[w_tiled][regular][rem]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       kBuffers * kStage);
-    if (e != hipSuccess) return e;
-    configured[w_tiled][regular][rem] = true;
-  }
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kBuffers * kStage); e != hipSuccess) return e;
   Plan p;
   p.a0 = an; p.a1 = as_; p.a2 = ao;
   p.b0 = bn; p.b1 = bs; p.b2 = bo;

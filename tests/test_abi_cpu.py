@@ -67,11 +67,43 @@ def test_validation_rejects_bad_shapes_before_any_launch(abi):
     assert "multiples of 32" in abi.status_string(10001)
 
 
+def test_validation_of_the_newer_entry_points(abi):
+    lib = abi.lib()
+    null = ctypes.c_void_p(0)
+    twelve = [null] * 12
+    assert lib.mg_padded_rows(0) == 0 and lib.mg_padded_rows(1) == 256 and lib.mg_padded_rows(256) == 256
+    assert lib.mg_padded_rows(4000) == 4096
+    assert lib.mg_weights_tileable(14336, 2560, 1408, 128) == 1
+    assert lib.mg_weights_tileable(4096, 8960, 4928, 448) == 0      # 4928 is not a multiple of 128
+    assert lib.mg_weights_tileable(1000, 2560, 1408, 128) == 0      # N not a multiple of 256
+    assert lib.mg_weights_tileable(256, 256, 0, 128) == 0           # an empty segment
+    # a_rows below M, unknown flag bits, tile-major flag on a shape that cannot be tiled
+    assert lib.mg_mixed_gemm_ex(*twelve, 8, 4, 256, 128, 128, 128, 0, null, null) == 10001
+    assert lib.mg_mixed_gemm_ex(*twelve, 8, 8, 256, 128, 128, 128, 2, null, null) == 10001
+    assert lib.mg_mixed_gemm_ex(*twelve, 8, 8, 256, 448, 416, 224, 1, null, null) == 10004
+    # tiling: N and the segment width must be whole tiles / stages; in place is refused
+    one = ctypes.c_void_p(256)
+    assert lib.mg_tile_weights(one, ctypes.c_void_p(512), 200, 128, null) == 10001
+    assert lib.mg_tile_weights(one, ctypes.c_void_p(512), 256, 96, null) == 10001
+    assert lib.mg_tile_weights(one, one, 256, 128, null) == 10002
+    assert lib.mg_tile_weights(null, null, 0, 128, null) == 0
+    # the normalising quantizer needs a weight vector and eps >= 0
+    six = [null] * 6
+    assert lib.mg_rmsnorm_reorder_quantize_x(null, null, 1e-5, null, 4, 4096, 2560, 1408, 128, *six, null) == 10002
+    assert lib.mg_rmsnorm_reorder_quantize_x(null, one, -1.0, null, 4, 4096, 2560, 1408, 128, *six, null) == 10001
+    # calibration
+    assert lib.mg_calibrate_reorder_index(null, 4, 100, null, null, 0, null) == 10001
+    assert lib.mg_calibrate_reorder_index(null, 4, 32768, null, null, 0, null) == 10004
+    assert lib.mg_calibrate_workspace_bytes(4096) >= 4096 * 4
+
+
 def test_fused_workspace_size(abi):
-    m, kn, ks, ko = 4096, 2560, 1408, 128
-    need = abi.fused_workspace_bytes(m, kn, ks, ko)
-    parts = [m * kn // 2, m * ks * 3 // 4, m * ko] + [mo.sf_bytes(m, k, "a") for k in (kn, ks, ko)]
-    assert need == sum((p + 255) // 256 * 256 for p in parts)
+    kn, ks, ko = 2560, 1408, 128
+    for m in (4096, 300, 8):      # sized for whole 256-row tiles
+        r = (m + 255) // 256 * 256
+        need = abi.fused_workspace_bytes(m, kn, ks, ko)
+        parts = [r * kn // 2, r * ks * 3 // 4, r * ko] + [mo.sf_bytes(r, k, "a") for k in (kn, ks, ko)]
+        assert need == sum((p + 255) // 256 * 256 for p in parts)
 
 
 def test_extension_module_surface():

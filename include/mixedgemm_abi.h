@@ -107,9 +107,11 @@ int mg_mixed_gemm_ex(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, c
 /* Rewrites one segment's weight codes src[N, kseg/2] (row-major, as mg_reorder_quantize_w wrote them;
  * the weight path of src/bindings.cpp:188-305) into tile-major order in dst (same size, dst != src):
  * per 256-feature tile and 128-wide K stage one block of 16 KB, ordered as the prefill kernel stages
- * it.  N a multiple of 256, kseg a multiple of 128.  Done once per layer, offline. */
+ * it; the 1-3 blocks of 32 a segment may have past its last whole stage follow as row-major rows.
+ * N a multiple of 256, kseg a multiple of 32.  Done once per layer, offline. */
 int mg_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, void* stream);
-/* 1 when weights of this shape can be tiled: N a multiple of 256, every segment a multiple of 128, none empty. */
+/* 1 when weights of this shape can be tiled: N a multiple of 256, every segment a multiple of 32 and
+ * at least 128 wide. */
 int mg_weights_tileable(int N, int KN, int KS, int KO);
 /* M rounded up to whole 256-token tiles. */
 int mg_padded_rows(int M);

@@ -99,11 +99,11 @@ int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, cons
 int mg_padded_rows(int M) { return M <= 0 ? 0 : (M + 255) / 256 * 256; }
 
 int mg_weights_tileable(int N, int KN, int KS, int KO) {
-  return N > 0 && N % 256 == 0 && KN >= 128 && KS >= 128 && KO >= 128 && (KN | KS | KO) % 128 == 0;
+  return N > 0 && N % 256 == 0 && KN >= 128 && KS >= 128 && KO >= 128 && (KN | KS | KO) % 32 == 0;
 }
 
 int mg_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, void* stream) {
-  if (N < 0 || kseg < 0 || N % 256 != 0 || kseg % 128 != 0) return MG_ERR_BAD_SHAPE;
+  if (N < 0 || kseg < 0 || N % 256 != 0 || kseg % 32 != 0) return MG_ERR_BAD_SHAPE;
   if (N == 0 || kseg == 0) return MG_OK;
   if (!ptr_ok(src, true) || !ptr_ok(dst, true) || src == dst) return MG_ERR_BAD_POINTER;
   return (int)mg::launch_tile_weights(src, dst, N, kseg, static_cast<hipStream_t>(stream));

@@ -201,10 +201,13 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
       const int xbytes = seg == 0 ? 16 : (seg == 1 ? 24 : 32);   // activation bytes per 32-element block
       const int left = nblk - 4 * q;
       const int gc = min(g, left - 1);
-      // tile-major weights: 16 KB per (256-feature tile, step), this workgroup's block in it, lane
-      // quad i, piece g; whole steps only
-      const size_t w_off = w_tiled ? ((((size_t)(blockIdx.x >> 4) * katoms + q) * 16 + (blockIdx.x & 15)) * 1024 + i * 64 + g * 16)
-                                   : ((size_t)nc * nblk * 16 + q * 64 + gc * 16);
+      // tile-major weights: 16 KB per (256-feature tile, whole step), this workgroup's block in it, lane
+      // quad i, piece g; the blocks past the last whole step as rows of (nblk % 4) blocks behind the tiled part
+      const int whole = nblk >> 2, rblk = nblk & 3;
+      const size_t w_tiled_off =
+          q < whole ? ((((size_t)(blockIdx.x >> 4) * whole + q) * 16 + (blockIdx.x & 15)) * 1024 + i * 64 + g * 16)
+                    : ((size_t)(N >> 8) * whole * 16384 + (size_t)nc * rblk * 16 + gc * 16);
+      const size_t w_off = w_tiled ? w_tiled_off : ((size_t)nc * nblk * 16 + q * 64 + gc * 16);
       wq[k] = *reinterpret_cast<const v4i*>(pb + w_off);
       sw[k] = psb[sf_offset(nc, 4 * q + gc, katoms)];
       // activations: two 16-byte pieces.  E2M1: block g (second piece unused);
@@ -621,8 +624,8 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
                              int a_rows, int N, int KN, int KS, int KO, unsigned flags, void* d, hipStream_t stream) {
   if (M == 0 || N == 0) return hipSuccess;
   const bool w_tiled = (flags & 1u) != 0;   // MG_FLAG_W_TILED
-  // tile-major weights exist only for shapes the 256x256 kernel takes, in whole stages
-  if (w_tiled && (!mixed_gemm_256_supported(256, N, KN, KS, KO) || (KN | KS | KO) % 128 != 0)) return hipErrorInvalidValue;
+  // tile-major weights exist only for shapes the 256x256 kernel takes
+  if (w_tiled && !mixed_gemm_256_supported(256, N, KN, KS, KO)) return hipErrorInvalidValue;
   const int m_pad = (M + 255) / 256 * 256;
   const int steps = (KN + 127) / 128 + (KS + 127) / 128 + (KO + 127) / 128;
   // whole 256-row tiles, the last one possibly reading rows past M (readable up to a_rows) and

@@ -637,12 +637,17 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a
 template <int FMT>
 __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                  const uint8_t* __restrict__ sfa, const uint8_t* __restrict__ sfb, int blk,
-                                                 const Ctx& c) {
+                                                 bool w_tiled, int tiles_n, const Ctx& c) {
   const int r = blk & 3, q = blk >> 2;
+  // weights: row-major rows of blk blocks, or (tile-major) the r blocks past the whole stages as rows of
+  // r blocks behind the tiled part; with r == 0 nothing is used and any valid address will do
+  const uint8_t* wbase = w_tiled ? (r ? b + (size_t)tiles_n * q * 16384 : b) : b;
+  const unsigned wpitch = w_tiled ? (unsigned)r * 16 : (unsigned)blk * 16;
+  const int wfirst = w_tiled ? 4 * q : 0;   // block index of the first block of a row
   constexpr int XB = Fmt<FMT>::row_bytes / 4;   // token bytes per block
   const int i = c.lane & 31, g = c.lane >> 5;
   const int katoms = (blk + 3) >> 2;
-  const unsigned ldb = (unsigned)blk * 16, lda = (unsigned)blk * XB;
+  const unsigned lda = (unsigned)blk * XB;
   const v4i z = {0, 0, 0, 0};
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -655,7 +660,7 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const unsigned n = c.n0 + c.wn * 128 + t * 32 + i, m = c.m0 + c.wm * 128 + t * 32 + i;
-      const v4i wv = *reinterpret_cast<const v4i*>(b + (size_t)n * ldb + (size_t)kbc * 16);
+      const v4i wv = *reinterpret_cast<const v4i*>(wbase + (size_t)n * wpitch + (size_t)max(kbc - wfirst, 0) * 16);
       const int sw = sfb[sf_offset(n, kbc, katoms)], sx = sfa[sf_offset(m, kbc, katoms)];
       f.w[t] = ok ? wv : z;
       sc.w[t] = ok ? sw : 127;
@@ -786,9 +791,9 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* 
 
   if constexpr (REM) {
     __builtin_amdgcn_sched_barrier(0);
-    remainder_blocks<kFmtE2M1>(acc, plan.a0, plan.b0, plan.sfa0, plan.sfb0, plan.blk0, c);
-    remainder_blocks<kFmtE3M2>(acc, plan.a1, plan.b1, plan.sfa1, plan.sfb1, plan.blk1, c);
-    remainder_blocks<kFmtE4M3>(acc, plan.a2, plan.b2, plan.sfa2, plan.sfb2, plan.blk2, c);
+    remainder_blocks<kFmtE2M1>(acc, plan.a0, plan.b0, plan.sfa0, plan.sfb0, plan.blk0, WT, tiles_n, c);
+    remainder_blocks<kFmtE3M2>(acc, plan.a1, plan.b1, plan.sfa1, plan.sfb1, plan.blk1, WT, tiles_n, c);
+    remainder_blocks<kFmtE4M3>(acc, plan.a2, plan.b2, plan.sfa2, plan.sfb2, plan.blk2, WT, tiles_n, c);
     __builtin_amdgcn_sched_barrier(0);
   }
 
@@ -845,13 +850,13 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
   const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
   const bool rem = (KN | KS | KO) % 128 != 0;
-  if (rem && w_tiled) return hipErrorInvalidValue;   // tile-major weights hold whole stages only
   typedef void (*kernel_t)(Plan, int, int, int, uint16_t*);
   // [tiled][regular][rem]
   const kernel_t kernels[2][2][2] = {
       {{mixed_gemm_256_kernel<false, false, false>, mixed_gemm_256_kernel<false, true, false>},
        {mixed_gemm_256_kernel<true, false, false>, mixed_gemm_256_kernel<true, true, false>}},
-      {{mixed_gemm_256_kernel<false, false, true>, nullptr}, {mixed_gemm_256_kernel<true, false, true>, nullptr}}};
+      {{mixed_gemm_256_kernel<false, false, true>, mixed_gemm_256_kernel<false, true, true>},
+       {mixed_gemm_256_kernel<true, false, true>, mixed_gemm_256_kernel<true, true, true>}}};
   const kernel_t kernel = kernels[w_tiled][regular][rem];
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kBuffers * kStage); e != hipSuccess) return e;
   Plan p;
@@ -869,27 +874,34 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   return hipGetLastError();
 }
 
-// Tile-major weight order of one segment (whole 128-wide stages, N a multiple of 256): per feature
-// tile of 256 rows and per stage one block of 16 KB, inside it the 16 copy blocks of 1 KB in the
-// order the kernel's LDS image wants them -- block j holds rows j + 16 * (2 * (k % 8) + k / 8) for
-// lane quad k = 0..15, 64 bytes (the stage's K range) each.  A copy instruction then reads 1 KB of
-// consecutive bytes (8 lines of 128 B) instead of 64 bytes from each of 16 rows (16 lines), and
-// the address unit, which limits the loop, has two thirds of the work.
+// Tile-major weight order of one segment (N a multiple of 256): per feature tile of 256 rows and per
+// whole 128-wide stage one block of 16 KB, inside it the 16 copy blocks of 1 KB in the order the
+// kernel's LDS image wants them -- block j holds rows j + 16 * (2 * (k % 8) + k / 8) for lane quad
+// k = 0..15, 64 bytes (the stage's K range) each.  A copy instruction then reads 1 KB of consecutive
+// bytes (8 lines of 128 B) instead of 64 bytes from each of 16 rows (16 lines), and the address
+// unit, which limits the loop, has two thirds of the work.  The 1-3 blocks of 32 elements a segment
+// may have past its last whole stage follow behind the tiled part as N row-major rows.
 __global__ void __launch_bounds__(256) tile_weights_kernel(const v4u* __restrict__ src, v4u* __restrict__ dst, int N, int blk) {
-  const size_t total = (size_t)N * blk;   // 16-byte units
-  const int nst = blk >> 2;
+  const int nst = blk >> 2, rem = blk & 3;
+  const size_t tiled = (size_t)N * nst * 4;   // 16-byte units in whole stages
+  const size_t total = (size_t)N * blk;
   for (size_t u = (size_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (size_t)gridDim.x * 256) {
-    const unsigned c = u & 3, k = (u >> 2) & 15, j = (u >> 6) & 15;
-    const size_t ts = u >> 10;   // tile_n * nst + stage
-    const unsigned ql = ts % nst;
-    const size_t tile_n = ts / nst;
-    const size_t row = tile_n * 256 + j + 16 * (2 * (k & 7) + (k >> 3));
-    dst[u] = src[row * blk + ql * 4 + c];
+    if (u < tiled) {
+      const unsigned c = u & 3, k = (u >> 2) & 15, j = (u >> 6) & 15;
+      const size_t ts = u >> 10;   // tile_n * nst + stage
+      const unsigned ql = ts % nst;
+      const size_t tile_n = ts / nst;
+      const size_t row = tile_n * 256 + j + 16 * (2 * (k & 7) + (k >> 3));
+      dst[u] = src[row * blk + ql * 4 + c];
+    } else {
+      const size_t v = u - tiled;
+      dst[u] = src[(v / rem) * blk + nst * 4 + v % rem];
+    }
   }
 }
 
 hipError_t launch_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, hipStream_t stream) {
-  if (N % 256 != 0 || kseg % 128 != 0) return hipErrorInvalidValue;
+  if (N % 256 != 0 || kseg % 32 != 0) return hipErrorInvalidValue;
   if (N == 0 || kseg == 0) return hipSuccess;
   const size_t units = (size_t)N * (kseg / 32);
   const int grid = (int)((units + 255) / 256 < 4096 ? (units + 255) / 256 : 4096);

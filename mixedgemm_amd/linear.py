@@ -88,7 +88,7 @@ class PackedWeights:
         if self.tiled:
             return self
         if not self.tileable():
-            raise ValueError("tile-major order needs N % 256 == 0 and three non-empty segments that are multiples of 128")
+            raise ValueError("tile-major order needs N % 256 == 0 and three segments of at least 128 channels")
         wn, ws, wo = abi.tile_weights(self.wn, self.ws, self.wo)
         return PackedWeights(wn, ws, wo, self.sfwn, self.sfws, self.sfwo, self.reorder_index, self.split, True)
 

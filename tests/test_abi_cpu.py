@@ -74,17 +74,18 @@ def test_validation_of_the_newer_entry_points(abi):
     assert lib.mg_padded_rows(0) == 0 and lib.mg_padded_rows(1) == 256 and lib.mg_padded_rows(256) == 256
     assert lib.mg_padded_rows(4000) == 4096
     assert lib.mg_weights_tileable(14336, 2560, 1408, 128) == 1
-    assert lib.mg_weights_tileable(4096, 8960, 4928, 448) == 0      # 4928 is not a multiple of 128
+    assert lib.mg_weights_tileable(4096, 8960, 4928, 448) == 1      # 32-granular segments are fine
+    assert lib.mg_weights_tileable(4096, 2560, 1408, 64) == 0       # a segment narrower than one stage
     assert lib.mg_weights_tileable(1000, 2560, 1408, 128) == 0      # N not a multiple of 256
     assert lib.mg_weights_tileable(256, 256, 0, 128) == 0           # an empty segment
     # a_rows below M, unknown flag bits, tile-major flag on a shape that cannot be tiled
     assert lib.mg_mixed_gemm_ex(*twelve, 8, 4, 256, 128, 128, 128, 0, null, null) == 10001
     assert lib.mg_mixed_gemm_ex(*twelve, 8, 8, 256, 128, 128, 128, 2, null, null) == 10001
-    assert lib.mg_mixed_gemm_ex(*twelve, 8, 8, 256, 448, 416, 224, 1, null, null) == 10004
+    assert lib.mg_mixed_gemm_ex(*twelve, 8, 8, 256, 448, 416, 64, 1, null, null) == 10004
     # tiling: N and the segment width must be whole tiles / stages; in place is refused
     one = ctypes.c_void_p(256)
     assert lib.mg_tile_weights(one, ctypes.c_void_p(512), 200, 128, null) == 10001
-    assert lib.mg_tile_weights(one, ctypes.c_void_p(512), 256, 96, null) == 10001
+    assert lib.mg_tile_weights(one, ctypes.c_void_p(512), 256, 100, null) == 10001
     assert lib.mg_tile_weights(one, one, 256, 128, null) == 10002
     assert lib.mg_tile_weights(null, null, 0, 128, null) == 0
     # the normalising quantizer needs a weight vector and eps >= 0

@@ -356,19 +356,21 @@ def test_whole_path_matches_golden_vectors(abi, path):
 
 # ------------------------------------------------------------------ tile-major weights
 def _tile_reference(w: np.ndarray) -> np.ndarray:
-    """Tile-major order of one segment's weight codes [N, kseg/2] (N % 256 == 0, kseg % 128 == 0):
-    [feature tile][stage][block j][lane quad k][64 bytes], row = 256 * tile + j + 16 * (2 * (k % 8) + k // 8)."""
+    """Tile-major order of one segment's weight codes [N, kseg/2] (N % 256 == 0, kseg % 32 == 0): whole
+    128-wide stages as [feature tile][stage][block j][lane quad k][64 bytes], row = 256 * tile + j +
+    16 * (2 * (k % 8) + k // 8); behind them what is left of every row, row-major."""
     n, cols = w.shape
     stages = cols // 64
-    v = w.reshape(n // 256, 256, stages, 64)
+    v = w[:, :stages * 64].reshape(n // 256, 256, stages, 64)
     k = np.arange(16)
     pr = 2 * (k % 8) + k // 8
     rows = (np.arange(16)[:, None] + 16 * pr[None, :])            # [j, k]
     out = v[:, rows, :, :]                                         # [tile, j, k, stage, 64]
-    return np.ascontiguousarray(out.transpose(0, 3, 1, 2, 4)).reshape(n, cols)
+    tiled = np.ascontiguousarray(out.transpose(0, 3, 1, 2, 4)).reshape(-1)
+    return np.concatenate([tiled, np.ascontiguousarray(w[:, stages * 64:]).reshape(-1)]).reshape(n, cols)
 
 
-@pytest.mark.parametrize("n,kseg", [(256, 128), (512, 384), (768, 2560)])
+@pytest.mark.parametrize("n,kseg", [(256, 128), (512, 384), (768, 2560), (256, 224), (512, 4928), (256, 160)])
 def test_tile_weights_matches_the_layout_formula(abi, n, kseg):
     rng = np.random.default_rng(n + kseg)
     w = rng.integers(0, 256, (n, kseg // 2), dtype=np.uint8)
@@ -387,6 +389,9 @@ TILED_SHAPES = [
     (256, 256, 128, 128, 128), (512, 512, 256, 384, 128), (256, 768, 2560, 1408, 128), (512, 256, 384, 512, 256),
     (300, 512, 2560, 1408, 128), (1000, 256, 384, 384, 384),
     (8, 512, 2560, 1408, 128), (20, 256, 128, 256, 128), (50, 768, 384, 128, 128), (130, 256, 2560, 896, 128),
+    # segments that end 32, 64 or 96 elements past their last whole stage (kept row-major behind the tiled part)
+    (256, 256, 448, 416, 224), (512, 512, 2240, 1248, 448), (300, 256, 160, 480, 352), (8, 256, 448, 416, 224),
+    (40, 512, 2240, 1248, 448),
 ]
 
 
@@ -418,8 +423,8 @@ def test_tiled_weights_give_the_same_result_bit_for_bit(abi, m, n, kn, ks, ko):
 
 def test_tiled_flag_is_refused_for_shapes_that_cannot_be_tiled(abi):
     from mixedgemm_amd.abi import MixedGemmError
-    assert not abi.weights_tileable(256, 448, 416, 224) and not abi.weights_tileable(200, 128, 128, 128)
-    m, n, kn, ks, ko = 16, 256, 448, 416, 224
+    assert not abi.weights_tileable(256, 448, 416, 64) and not abi.weights_tileable(200, 128, 128, 128)
+    m, n, kn, ks, ko = 16, 256, 448, 416, 64
     x = H.make_activations(m, kn + ks + ko, 3).to(DEV)
     idx = H.random_index(kn + ks + ko, 4).to(DEV)
     aq = abi.reorder_quantize_x(x, idx, kn, ks, ko)

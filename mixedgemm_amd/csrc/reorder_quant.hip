@@ -13,6 +13,8 @@
 // 32-element block (no cross-lane reduction), the scale exponent comes from
 // integer arithmetic on the float bits, and the element conversion is done by
 // the gfx950 cvt_scalef32 instructions on the already integer-rounded values.
+#include <type_traits>
+
 #include "mg_common.h"
 
 namespace mg {
@@ -50,7 +52,7 @@ __device__ __forceinline__ void quantize_store(const float (&f)[32], int fmt, ui
                                                uint8_t* __restrict__ sf) {
   float amax = 0.0f;
 #pragma unroll
-  for (int p = 0; p < 32; p += 2) amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(f[p]), __builtin_fabsf(f[p + 1])));
+  for (int p = 0; p < 32; p += 2) amax = __builtin_fmaxf(__builtin_fmaxf(amax, __builtin_fabsf(f[p])), __builtin_fabsf(f[p + 1]));
   const int byte = scale_byte(amax, fmt);
   const float rs = __uint_as_float((unsigned)(254 - byte) << 23);
   float v[32];
@@ -175,9 +177,22 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
     for (int it = 0; it < 4; ++it)
       gv[it] = *reinterpret_cast<const v4u*>(gamma + (size_t)min(tid + it * nthr, nchunks - 1) * 8);
   }
-  int parity = 0;
-  for (; group < ngroups; group += gridDim.x, parity ^= 1) {
-    uint8_t* lds = lds_all + parity * buf_stride;
+  // Byte offsets of the lane's 32 gathered channels inside a tile (the same for every row).
+  unsigned ga[32];
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      ga[q * 8 + e] = ((e & 1) ? (iv[q][e >> 1] >> 16) : (iv[q][e >> 1] & 0xffffu)) * (2 * R);
+
+  // The loop body exists once per LDS buffer, so that the buffer's offset is a compile-time
+  // constant wherever the buffers are a fixed distance apart (kFixed) and folds into the LDS
+  // instructions' immediate offsets: the gather is then one instruction per channel.
+  constexpr bool kFixed = MAXT == 256;
+  constexpr int kBuf1 = MAXT * 64 * R;   // largest tile of this instantiation
+  auto body = [&](auto parity_c) {
+    constexpr int parity = decltype(parity_c)::value;
+    uint8_t* lds = lds_all + (kFixed ? parity * kBuf1 : parity * buf_stride);
     const int row0 = group * R;
     if constexpr (NORM) {
       double ss[R];
@@ -261,16 +276,15 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
       for (int q = 0; q < 4; ++q) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const unsigned ch = (e & 1) ? (iv[q][e >> 1] >> 16) : (iv[q][e >> 1] & 0xffffu);
           const int p = q * 8 + e;
           if constexpr (R == 4) {
-            const v2u d = *reinterpret_cast<const v2u*>(lds + ch * 8);
+            const v2u d = *reinterpret_cast<const v2u*>(lds + ga[p]);
             g[p][0] = d[0];
             g[p][1] = d[1];
           } else if constexpr (R == 2) {
-            g[p][0] = *reinterpret_cast<const unsigned*>(lds + ch * 4);
+            g[p][0] = *reinterpret_cast<const unsigned*>(lds + ga[p]);
           } else {
-            g[p][0] = *reinterpret_cast<const uint16_t*>(lds + ch * 2);
+            g[p][0] = *reinterpret_cast<const uint16_t*>(lds + ga[p]);
           }
         }
       }
@@ -290,6 +304,14 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
     }
     // with one buffer (buf_stride == 0) there is exactly one group per workgroup; with two, the
     // barrier of the next iteration separates this gather from the stores two iterations on
+  };
+  while (true) {
+    body(std::integral_constant<int, 0>{});
+    group += gridDim.x;
+    if (group >= ngroups) break;
+    body(std::integral_constant<int, 1>{});
+    group += gridDim.x;
+    if (group >= ngroups) break;
   }
 }
 
@@ -313,12 +335,14 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
 #ifndef MG_QUANT_WGS_PER_CU
 #define MG_QUANT_WGS_PER_CU 4
 #endif
-    int per_cu = (160 * 1024) / (2 * tile);
+    // second LDS buffer: a fixed 16 KB * R behind the first for the 256-lane kernels (see kFixed), else one tile behind
+    const int second = K <= 8192 ? 256 * 64 * R : tile;
+    int per_cu = (160 * 1024) / (second + tile);
     per_cu = per_cu < 1 ? 1 : (per_cu > MG_QUANT_WGS_PER_CU ? MG_QUANT_WGS_PER_CU : per_cu);
     const int resident = 256 * per_cu;
-    const bool stream_groups = ngroups > resident && 2 * tile <= 160 * 1024;
+    const bool stream_groups = ngroups > resident && second + tile <= 160 * 1024;
     const int grid = stream_groups ? resident : ngroups;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), (size_t)(stream_groups ? 2 * tile : tile), stream, xb, idx, rows, K,
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), (size_t)(stream_groups ? second + tile : tile), stream, xb, idx, rows, K,
                        KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream_groups ? tile : 0, gm, eps);
   };
 #ifndef MG_QUANT_R_SMALLK

@@ -19,6 +19,8 @@
 //                [64+16g, 64+16g+16) in registers 4-7 (two 16-byte pieces);
 // and, for every format, the E8M0 scale of block g of row i in the byte of the
 // scale register that op_sel selects.
+#include <stdlib.h>
+
 #include "mg_common.h"
 
 namespace mg {
@@ -158,35 +160,45 @@ __device__ __forceinline__ v4f decode_mfma(v8i wb, v8i xa, v4f acc, int sw, int 
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wb, xa, acc, kFmtE2M1, FMT, 0, sw, 0, sx);
 }
 
-template <int G>
+template <int G, int F>
 __global__ void __launch_bounds__(256)
 mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, int M, int N, int steps_per_wave,
                          int w_tiled, uint16_t* __restrict__ d) {
-  constexpr int S = G >= 8 ? 1 : 8 / G;   // K steps a wave keeps in flight at once
-  __shared__ float partial[4][G][16 * 16];
+  constexpr int S = G * F >= 8 ? 1 : 8 / (G * F);   // K steps a wave keeps in flight at once
+  __shared__ float partial[4][F][G][16 * 16];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, g = lane >> 4;
-  // Row-major weights: the workgroup owns 16 consecutive features.  Tile-major weights: the 16 rows
-  // of one 1 KB copy block (block j = blockIdx.x % 16 of feature tile blockIdx.x / 16), i.e. features
+  // The workgroup owns F groups of 16 features (group index bx = blockIdx.x * F + f) and G groups of 16
+  // tokens; an activation fragment is loaded once and used for the F feature groups.
+  // Row-major weights: a group is 16 consecutive features.  Tile-major weights: the 16 rows of one
+  // 1 KB copy block (block j = bx % 16 of feature tile bx / 16), i.e. features
   // j + 16 * (2 * (t % 8) + t / 8) of the tile for t = 0..15, so that a weight load reads 1 KB of
   // consecutive bytes.
-  const int tile_row0 = (blockIdx.x >> 4) * 256 + (blockIdx.x & 15);
-  const int n = w_tiled ? tile_row0 + 16 * (2 * (i & 7) + (i >> 3)) : blockIdx.x * 16 + i;
-  const int m0 = m_base + blockIdx.y * (G * 16) + i;      // this lane's token in group 0
-  const bool n_ok = n < N;
-  const int nc = min(n, N - 1);   // clamped rows: every load is in bounds and unconditional
-  const int total = s4.steps + s6.steps + s8.steps;
-  v4f acc[G];
+  int tile_row0[F], n[F], nc[F];
+  bool n_ok[F];
 #pragma unroll
-  for (int gi = 0; gi < G; ++gi) acc[gi] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int f = 0; f < F; ++f) {
+    const int bx = blockIdx.x * F + f;
+    tile_row0[f] = (bx >> 4) * 256 + (bx & 15);
+    n[f] = w_tiled ? tile_row0[f] + 16 * (2 * (i & 7) + (i >> 3)) : bx * 16 + i;
+    n_ok[f] = n[f] < N;
+    nc[f] = min(n[f], N - 1);   // clamped rows: every load is in bounds and unconditional
+  }
+  const int m0 = m_base + blockIdx.y * (G * 16) + i;      // this lane's token in group 0
+  const int total = s4.steps + s6.steps + s8.steps;
+  v4f acc[F][G];
+#pragma unroll
+  for (int f = 0; f < F; ++f)
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) acc[f][gi] = v4f{0.f, 0.f, 0.f, 0.f};
 
   for (int r0 = 0; r0 < steps_per_wave; r0 += S) {
     const int t0 = wave * steps_per_wave + r0, t_end = min(total, wave * steps_per_wave + steps_per_wave);
 
     // Straight-line issue of every load of this round, so all of them are in
     // flight together; masking comes afterwards.
-    v4i wq[S], xa[S][G], xb[S][G];
-    int sw[S], sx[S][G];
+    v4i wq[S][F], xa[S][G], xb[S][G];
+    int sw[S][F], sx[S][G];
 #pragma unroll
     for (int k = 0; k < S; ++k) {
       const int t = min(t0 + k, total - 1);
@@ -201,15 +213,19 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
       const int xbytes = seg == 0 ? 16 : (seg == 1 ? 24 : 32);   // activation bytes per 32-element block
       const int left = nblk - 4 * q;
       const int gc = min(g, left - 1);
-      // tile-major weights: 16 KB per (256-feature tile, whole step), this workgroup's block in it, lane
+      // tile-major weights: 16 KB per (256-feature tile, whole step), the group's block in it, lane
       // quad i, piece g; the blocks past the last whole step as rows of (nblk % 4) blocks behind the tiled part
       const int whole = nblk >> 2, rblk = nblk & 3;
-      const size_t w_tiled_off =
-          q < whole ? ((((size_t)(blockIdx.x >> 4) * whole + q) * 16 + (blockIdx.x & 15)) * 1024 + i * 64 + g * 16)
-                    : ((size_t)(N >> 8) * whole * 16384 + (size_t)nc * rblk * 16 + gc * 16);
-      const size_t w_off = w_tiled ? w_tiled_off : ((size_t)nc * nblk * 16 + q * 64 + gc * 16);
-      wq[k] = *reinterpret_cast<const v4i*>(pb + w_off);
-      sw[k] = psb[sf_offset(nc, 4 * q + gc, katoms)];
+#pragma unroll
+      for (int f = 0; f < F; ++f) {
+        const int bx = blockIdx.x * F + f;
+        const size_t w_tiled_off =
+            q < whole ? ((((size_t)(bx >> 4) * whole + q) * 16 + (bx & 15)) * 1024 + i * 64 + g * 16)
+                      : ((size_t)(N >> 8) * whole * 16384 + (size_t)nc[f] * rblk * 16 + gc * 16);
+        const size_t w_off = w_tiled ? w_tiled_off : ((size_t)nc[f] * nblk * 16 + q * 64 + gc * 16);
+        wq[k][f] = *reinterpret_cast<const v4i*>(pb + w_off);
+        sw[k][f] = psb[sf_offset(nc[f], 4 * q + gc, katoms)];
+      }
       // activations: two 16-byte pieces.  E2M1: block g (second piece unused);
       // E3M2: bytes [0,16) and [8,24) of block g; E4M3: K [16g,+16) and [64+16g,+16).
       const int a_blk = seg == 2 ? (g >> 1) : g, b_blk = seg == 2 ? 2 + (g >> 1) : g;
@@ -236,11 +252,16 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
         const int nblk = seg == 0 ? s4.nblk : (seg == 1 ? s6.nblk : s8.nblk);
         const int left = nblk - 4 * q;
         const bool blk_ok = g < left;
-        const bool w_ok = n_ok && blk_ok;
         const v4i z = {0, 0, 0, 0};
-        const v4i w4 = w_ok ? wq[k] : z;
-        const v8i wf = {w4[0], w4[1], w4[2], w4[3], 0, 0, 0, 0};
-        const int s_w = w_ok ? sw[k] : 127;
+        v8i wf[F];
+        int s_w[F];
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+          const bool w_ok = n_ok[f] && blk_ok;
+          const v4i w4 = w_ok ? wq[k][f] : z;
+          wf[f] = v8i{w4[0], w4[1], w4[2], w4[3], 0, 0, 0, 0};
+          s_w[f] = w_ok ? sw[k][f] : 127;
+        }
 #pragma unroll
         for (int gi = 0; gi < G; ++gi) {
           const bool m_ok = m0 + gi * 16 < M;
@@ -248,17 +269,20 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
           if (seg == 0) {
             const v4i a4 = (m_ok && blk_ok) ? xa[k][gi] : z;
             const v8i xf = {a4[0], a4[1], a4[2], a4[3], 0, 0, 0, 0};
-            acc[gi] = decode_mfma<kFmtE2M1>(wf, xf, acc[gi], s_w, s_x);
+#pragma unroll
+            for (int f = 0; f < F; ++f) acc[f][gi] = decode_mfma<kFmtE2M1>(wf[f], xf, acc[f][gi], s_w[f], s_x);
           } else if (seg == 1) {
             const v4i a4 = (m_ok && blk_ok) ? xa[k][gi] : z;
             const v4i b4 = (m_ok && blk_ok) ? xb[k][gi] : z;
             const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4[2], b4[3], 0, 0};
-            acc[gi] = decode_mfma<kFmtE3M2>(wf, xf, acc[gi], s_w, s_x);
+#pragma unroll
+            for (int f = 0; f < F; ++f) acc[f][gi] = decode_mfma<kFmtE3M2>(wf[f], xf, acc[f][gi], s_w[f], s_x);
           } else {
             const v4i a4 = (m_ok && (g >> 1) < left) ? xa[k][gi] : z;
             const v4i b4 = (m_ok && 2 + (g >> 1) < left) ? xb[k][gi] : z;
             const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4[0], b4[1], b4[2], b4[3]};
-            acc[gi] = decode_mfma<kFmtE4M3>(wf, xf, acc[gi], s_w, s_x);
+#pragma unroll
+            for (int f = 0; f < F; ++f) acc[f][gi] = decode_mfma<kFmtE4M3>(wf[f], xf, acc[f][gi], s_w[f], s_x);
           }
         }
       }
@@ -267,24 +291,27 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
 
   // result tile is D^T: lane holds token m = lane % 16, features 4 * (lane / 16) + v
 #pragma unroll
-  for (int gi = 0; gi < G; ++gi) *reinterpret_cast<v4f*>(&partial[wave][gi][lane * 4]) = acc[gi];
-  __syncthreads();
-  // wave w sums and writes groups w, w + 4, ...
+  for (int f = 0; f < F; ++f)
 #pragma unroll
-  for (int gi = 0; gi < G; ++gi) {
-    if ((gi & 3) != wave && G >= 4) continue;
-    if (G < 4 && wave != gi) continue;
+    for (int gi = 0; gi < G; ++gi) *reinterpret_cast<v4f*>(&partial[wave][f][gi][lane * 4]) = acc[f][gi];
+  __syncthreads();
+  // the F * G partial tiles are dealt to the 4 waves round-robin
+#pragma unroll
+  for (int fg = 0; fg < F * G; ++fg) {
+    if ((fg & 3) != wave) continue;
+    const int f = fg / G, gi = fg % G;
     v4f sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < 4; ++w) sum += *reinterpret_cast<const v4f*>(&partial[w][gi][lane * 4]);
-    const int nn = blockIdx.x * 16 + 4 * g;
+    for (int w = 0; w < 4; ++w) sum += *reinterpret_cast<const v4f*>(&partial[w][f][gi][lane * 4]);
+    const int nn = (blockIdx.x * F + f) * 16 + 4 * g;
     const int m = m0 + gi * 16;
     if (m < M) {
-      if (w_tiled) {   // feature 4g + v of the workgroup is row tile_row0 + 16 * (2 * (t % 8) + t / 8), t = 4g + v
+      if (w_tiled) {   // feature 4g + v of the group is row tile_row0 + 16 * (2 * (t % 8) + t / 8), t = 4g + v
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           const int t = 4 * g + v;
-          d[(size_t)m * N + tile_row0 + 16 * (2 * (t & 7) + (t >> 3))] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
+          const int row = tile_row0[f] + 16 * (2 * (t & 7) + (t >> 3));
+          if (row < N) d[(size_t)m * N + row] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
         }
       } else {
         uint16_t* dst = d + (size_t)m * N + nn;
@@ -296,18 +323,40 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
   }
 }
 
+// Feature groups of 16 per workgroup of the skinny kernel.
+static int skinny_feature_groups(int rows, int N) {
+  const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
+  return ceil_div(N, 32) * ceil_div(rows, 16 * g) >= 256 ? 2 : 1;
+}
+
 hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int m_base, int M, int N,
                          bool w_tiled, uint16_t* d, hipStream_t stream) {
   const int rows = M - m_base;
   const int steps_per_wave = (d4.steps + d6.steps + d8.steps + 3) / 4;
   const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
-  const dim3 grid(ceil_div(N, 16), ceil_div(rows, 16 * g));
+  // two feature groups per workgroup for 17-64 tokens: each activation fragment then serves 32 features
+  // two feature groups per workgroup (an activation fragment then serves 32 features) as long as that
+  // leaves a workgroup for every CU; measured on N = 2048 ... 14336
+  const int f = skinny_feature_groups(rows, N);
+  const dim3 grid(ceil_div(N, 16 * f), ceil_div(rows, 16 * g));
   const int wt = w_tiled ? 1 : 0;
   switch (g) {
-    case 1: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<1>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d); break;
-    case 2: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<2>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d); break;
-    case 4: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<4>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d); break;
-    default: hipLaunchKernelGGL(mixed_gemm_skinny_kernel<8>, grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d); break;
+    case 1:
+      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<1, 2>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<1, 1>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      break;
+    case 2:
+      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<2, 2>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<2, 1>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      break;
+    case 4:
+      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<4, 2>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<4, 1>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      break;
+    default:
+      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<8, 2>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<8, 1>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      break;
   }
   return hipGetLastError();
 }
@@ -607,14 +656,15 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
 
 // Rough launch times in microseconds (measured on MI355X, K = 4096: a 128-wide stage takes ~1.05 us
 // with every CU busy and ~0.7 us when at most half of them are, plus ~8 us of fill and drain per
-// round of 256 tiles; 0.28 ns per 16 tokens x 16 features x 128 K on the skinny kernel), only to
+// round of 256 tiles; 0.19-0.25 ns per 16 tokens x 16 features x 128 K on the skinny kernel), only to
 // choose between the two for fewer than 256 tokens.
 static double pipelined_us(int m_pad, int N, int stages) {
   const int tiles = (m_pad / 256) * (N / 256);
   return (double)((tiles + 255) / 256) * (stages * (tiles <= 128 ? 0.7 : 1.05) + 8.0);
 }
 static double skinny_us(int rows, int N, int steps) {
-  return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * 0.28e-3;
+  const double per_unit = skinny_feature_groups(rows, N) == 2 ? 0.19e-3 : 0.25e-3;
+  return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * per_unit;
 }
 
 // a_rows: token rows for which the activation codes and scales are readable (>= M)

@@ -120,6 +120,26 @@ def _rows_view(alloc_rows, rows, cols, **kw):
     return torch.empty((alloc_rows, cols), **kw)[:rows]
 
 
+def _check_out(out, shape, dtype, name):
+    """A caller-provided output must be what the call would have allocated."""
+    _require(out, dtype, name)
+    if tuple(out.shape) != tuple(shape):
+        raise MixedGemmError(f"{name}: expected shape {tuple(shape)}, got {tuple(out.shape)}")
+
+
+def _check_quant_out(out, rows, kn, ks, ko, operand):
+    if len(out) != 6:
+        raise MixedGemmError("out: expected six tensors (codes x3, scales x3)")
+    w = operand == MG_OPERAND_B
+    shapes = ((rows, kn // 2), (rows, ks // 2 if w else ks // 4 * 3), (rows, ko // 2 if w else ko))
+    for t, shape, name in zip(out[:3], shapes, ("qn", "qs", "qo")):
+        _check_out(t, shape, torch.uint8, name)
+    for t, kseg, name in zip(out[3:], (kn, ks, ko), ("sfn", "sfs", "sfo")):
+        _require(t, torch.uint8, name)
+        if t.numel() < sf_bytes(rows, kseg, operand):
+            raise MixedGemmError(f"{name}: {t.numel()} bytes, need {sf_bytes(rows, kseg, operand)}")
+
+
 def alloc_quant_outputs(rows, kn, ks, ko, operand, device):
     """The six output tensors of a reorder-quantize call (codes x3, scales x3), with the
     reference's shapes.  For activations the storage behind them has room for whole 256-row
@@ -150,6 +170,8 @@ def _reorder_quantize(fn_name, operand, t, idx, kn, ks, ko, out=None):
         raise MixedGemmError(f"reorder_index has {idx.numel()} entries, input has {k} channels")
     if out is None:
         out = alloc_quant_outputs(rows, kn, ks, ko, operand, t.device)
+    else:
+        _check_quant_out(out, rows, kn, ks, ko, operand)
     qn, qs, qo, sfn, sfs, sfo = out
     status = getattr(lib(), fn_name)(_ptr(t), _ptr(idx), rows, k, kn, ks, ko,
                                      _ptr(qn), _ptr(qs), _ptr(qo), _ptr(sfn), _ptr(sfs), _ptr(sfo), _stream(t))
@@ -174,6 +196,8 @@ def rmsnorm_reorder_quantize_x(x, norm_weight, eps, reorder_index, kn, ks, ko, o
         raise MixedGemmError(f"reorder_index / norm_weight must have {k} entries")
     if out is None:
         out = alloc_quant_outputs(rows, kn, ks, ko, MG_OPERAND_A, x.device)
+    else:
+        _check_quant_out(out, rows, kn, ks, ko, MG_OPERAND_A)
     qn, qs, qo, sfn, sfs, sfo = out
     check(lib().mg_rmsnorm_reorder_quantize_x(_ptr(x), _ptr(norm_weight), float(eps), _ptr(reorder_index), rows, k, kn, ks,
                                               ko, _ptr(qn), _ptr(qs), _ptr(qo), _ptr(sfn), _ptr(sfs), _ptr(sfo),
@@ -196,6 +220,12 @@ def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None
     kn, ks, ko = an.shape[1] * 2, as_.shape[1] * 4 // 3, ao.shape[1]
     if out is None:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=an.device)
+    else:
+        _check_out(out, (m, n), torch.bfloat16, "out")
+    if bs.shape[0] != n or bo.shape[0] != n or as_.shape[0] != m or ao.shape[0] != m:
+        raise MixedGemmError("the three segments of an operand must have the same number of rows")
+    if bn.shape[1] * 2 != kn or bs.shape[1] * 2 != ks or bo.shape[1] * 2 != ko:
+        raise MixedGemmError("activation and weight segments disagree on KN / KS / KO")
     # rows the activation buffers are readable for: whole tiles if every storage has the room
     r = padded_rows(m)
     roomy = all(_capacity(t) >= r * t.shape[1] for t in (an, as_, ao)) and all(
@@ -220,6 +250,12 @@ def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, wor
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    else:
+        _check_out(out, (m, n), torch.bfloat16, "out")
+    if x.shape[1] != kn + ks + ko or reorder_index.numel() != x.shape[1]:
+        raise MixedGemmError(f"X has {x.shape[1]} channels, the split sums to {kn + ks + ko}, the index has {reorder_index.numel()}")
+    if workspace.numel() < need or not workspace.is_cuda or workspace.dtype != torch.uint8:
+        raise MixedGemmError(f"workspace: need {need} uint8 on the GPU")
     if norm_weight is not None:
         _require(norm_weight, torch.bfloat16, "norm_weight")
         if norm_weight.numel() != x.shape[1]:
@@ -259,6 +295,10 @@ def calibrate_reorder_index(x, out=None, workspace=None):
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty(k, dtype=torch.int16, device=x.device)
+    else:
+        _check_out(out, (k,), torch.int16, "out")
+    if workspace.numel() < need or not workspace.is_cuda:
+        raise MixedGemmError(f"workspace: need {need} bytes on the GPU")
     check(lib().mg_calibrate_reorder_index(_ptr(x), m, k, _ptr(out), _ptr(workspace), workspace.numel(),
                                            _stream(x)), "mg_calibrate_reorder_index")
     return out

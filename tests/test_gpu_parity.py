@@ -471,3 +471,43 @@ def test_fused_norm_linear_equals_norm_then_linear(abi):
     assert torch.equal(d1, d2)
     qx, qw = _oracle_operands(y, w, idx, kn, ks, ko)
     _check_gemm(d1, qx, qw, "fused norm linear")
+
+
+# ------------------------------------------------------------------ host-side argument checks and empty problems
+def test_wrong_outputs_and_mismatched_operands_are_refused(abi):
+    from mixedgemm_amd.abi import MixedGemmError
+    m, n, kn, ks, ko = 8, 32, 128, 128, 128
+    k = kn + ks + ko
+    x = H.make_activations(m, k, 1).to(DEV)
+    idx = H.random_index(k, 2).to(DEV)
+    aq = abi.reorder_quantize_x(x, idx, kn, ks, ko)
+    bq = abi.reorder_quantize_w(H.make_weights(n, k, 3).to(DEV), idx, kn, ks, ko)
+    args = (aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5])
+    with pytest.raises(MixedGemmError):
+        abi.matmul(*args, out=torch.empty((m, n + 1), dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(MixedGemmError):
+        abi.matmul(*args, out=torch.empty((m, n), dtype=torch.float16, device=DEV))
+    with pytest.raises(MixedGemmError):     # weights quantized with another split
+        b2 = abi.reorder_quantize_w(H.make_weights(n, k, 3).to(DEV), idx, 256, 64, 64)
+        abi.matmul(aq[0], b2[0], aq[1], b2[1], aq[2], b2[2], aq[3], b2[3], aq[4], b2[4], aq[5], b2[5])
+    with pytest.raises(MixedGemmError):
+        abi.reorder_quantize_x(x, idx, kn, ks, ko, out=aq[:5])
+    with pytest.raises(MixedGemmError):
+        abi.fused_linear(x, idx, *bq, kn, ks, ko, workspace=torch.empty(16, dtype=torch.uint8, device=DEV))
+    with pytest.raises(MixedGemmError):
+        abi.reorder_quantize_x(x, idx[:-1].contiguous(), kn, ks, ko)
+
+
+def test_empty_problems(abi):
+    kn, ks, ko = 128, 128, 128
+    k = kn + ks + ko
+    idx = H.random_index(k, 2).to(DEV)
+    x0 = torch.empty((0, k), dtype=torch.bfloat16, device=DEV)
+    aq = abi.reorder_quantize_x(x0, idx, kn, ks, ko)
+    assert aq[0].shape == (0, kn // 2)
+    bq = abi.reorder_quantize_w(H.make_weights(32, k, 3).to(DEV), idx, kn, ks, ko)
+    d = abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5])
+    assert d.shape == (0, 32)
+    d = abi.fused_linear(x0, idx, *bq, kn, ks, ko)
+    torch.cuda.synchronize()
+    assert d.shape == (0, 32)

@@ -6,6 +6,7 @@
 Outputs (kept out of git, shipped with the tree):
     mixedgemm_amd/lib/libmixedgemm_hip.so   hand-written gfx950 kernels + extern "C" entry points
     build/mixedgemm.so                      torch extension with the reference's operator surface
+    build/abi_driver                        torch-free host program (tests/c_host) on the C-ABI
 """
 from __future__ import annotations
 
@@ -21,6 +22,8 @@ LIB_DIR = os.path.join(PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmixedgemm_hip.so")
 EXT_DIR = os.path.join(ROOT, "build")
 EXT_PATH = os.path.join(EXT_DIR, "mixedgemm.so")
+DRIVER_SRC = os.path.join(ROOT, "tests", "c_host", "abi_driver.cpp")
+DRIVER_PATH = os.path.join(EXT_DIR, "abi_driver")
 
 HIP_SOURCES = ["abi.hip", "reorder_quant.hip", "mixed_gemm.hip", "mixed_gemm_256.hip", "calibrate.hip", "ceiling.hip"]
 HIP_HEADERS = ["mg_common.h", os.path.join(ROOT, "include", "mixedgemm_abi.h")]
@@ -80,9 +83,23 @@ def build_torch_extension(force: bool = False, verbose: bool = False) -> str:
     return EXT_PATH
 
 
+def build_c_host_driver(force: bool = False, verbose: bool = False) -> str:
+    """The torch-free host program of tests/c_host (HIP runtime + the C-ABI only)."""
+    deps = [DRIVER_SRC, os.path.join(ROOT, "include", "mixedgemm_abi.h"), LIB_PATH]
+    if force or _stale(DRIVER_PATH, deps):
+        os.makedirs(EXT_DIR, exist_ok=True)
+        cmd = ["hipcc", "-O2", "-std=c++17", f"-I{os.path.join(ROOT, 'include')}", DRIVER_SRC, "-o", DRIVER_PATH,
+               f"-L{LIB_DIR}", "-lmixedgemm_hip", f"-Wl,-rpath,{LIB_DIR}", "-Wl,-rpath,$ORIGIN/../mixedgemm_amd/lib"]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+    return DRIVER_PATH
+
+
 def build_all(force: bool = False, verbose: bool = False) -> None:
     build_hip_library(force, verbose)
     build_torch_extension(force, verbose)
+    build_c_host_driver(force, verbose)
 
 
 if __name__ == "__main__":

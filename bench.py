@@ -326,7 +326,7 @@ def main():
         from oracle import mx_oracle as mo
         from oracle import scalar as sc
         torch_threads = torch.get_num_threads()
-        rows = 256
+        rows = m          # the whole c3 workload: a step takes the host cores well under a second
         wq_host = sc.quantize_w(H.bf16_bits(w), idx.numpy(), kn, ks, ko)          # offline, as on the GPU
         wdeq = torch.from_numpy(np.concatenate([
             mo.dequantize(mo.unpack_fp4(wq_host[q]), mo.sf_gather(wq_host[s], n, kk), "e2m1")
@@ -342,7 +342,7 @@ def main():
             return (torch.from_numpy(xdeq) @ wdeq.T).to(torch.bfloat16)
 
         cpu_step()
-        reps = 3
+        reps = 30
         c0 = time.perf_counter()
         for _ in range(reps):
             cpu_step()
@@ -350,24 +350,26 @@ def main():
         cpu = {
             "value": round(2.0 * rows * n * k / c_s / 1e12, 4), "unit": "TFLOP/s",
             "cores": torch_threads, "kind": "port",
-            "sample": f"first {rows} of {m} token rows of c3 (full N={n}, K={k}): C-oracle reorder-quantize + NumPy "
-                      f"dequantize + torch fp32 matmul, weights quantized offline; 1 warm-up + {reps} repeats; "
-                      f"os.cpu_count()={os.cpu_count()}",
+            "sample": f"all {rows} token rows of c3 (N={n}, K={k}): C-oracle reorder-quantize + NumPy "
+                      f"dequantize + torch fp32 matmul, weights quantized offline; 1 warm-up + {reps} repeats "
+                      f"({c_s * reps:.1f} s of host work); os.cpu_count()={os.cpu_count()}",
         }
         if "reorder_quant_c1" in extra:
             m1, _, k1, kn1, ks1, ko1 = H.CONFIGS["c1"]
-            r1 = 1024
+            r1 = m1
+            reps1 = 500
             x1b = H.bf16_bits(H.make_activations(m1, k1, 1234 + 1)[:r1])
             i1 = H.random_index(k1, 4321).numpy()
             sc.quantize_x(x1b, i1, kn1, ks1, ko1)
             c0 = time.perf_counter()
-            for _ in range(reps):
+            for _ in range(reps1):
                 sc.quantize_x(x1b, i1, kn1, ks1, ko1)
-            c1_s = (time.perf_counter() - c0) / reps
+            c1_s = (time.perf_counter() - c0) / reps1
             extra["reorder_quant_c1"]["cpu_baseline"] = {
                 "value": round(quant_bytes(r1, k1, kn1, ks1, ko1) / c1_s / 1e9, 3), "unit": "GB/s",
                 "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count())), "kind": "port",
-                "sample": f"first {r1} of {m1} rows of c1, scalar C oracle with OpenMP over rows",
+                "sample": f"all {r1} rows of c1, scalar C oracle with OpenMP over rows, {reps1} repeats "
+                          f"({c1_s * reps1:.1f} s of host work)",
             }
 
     out = {

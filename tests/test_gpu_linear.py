@@ -136,3 +136,43 @@ def test_layer_with_fused_rmsnorm(linear):
     torch.cuda.synchronize()
     ref, slack = _oracle_linear(y, w, idx, split)
     _close(out, ref, slack)
+
+
+def test_layer_replayed_as_a_hip_graph(linear):
+    """The whole layer (RMSNorm + reorder-quantize + GEMM: three of our launches, nothing else) captured once
+    and replayed with new inputs in the same buffers; every replay must equal the eager result."""
+    m, n, k = 300, 512, 4096
+    split = linear.default_split(k)
+    g = torch.Generator().manual_seed(7)
+    gamma = (torch.randn(k, generator=g) * 0.3 + 1.0).to(torch.bfloat16).to(DEV)
+    xs = [H.make_activations(m, k, 200 + i).to(DEV) for i in range(3)]
+    w = H.make_weights(n, k, 210).to(DEV)
+    from mixedgemm_amd import abi
+    idx = abi.calibrate_reorder_index(xs[0])
+    pw = linear.PackedWeights.from_float(w, idx, split)
+    x_buf = xs[0].clone()
+    ws = torch.empty(abi.fused_workspace_bytes(m, *split), dtype=torch.uint8, device=DEV)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+
+    def run():
+        abi.fused_linear(x_buf, idx, *pw.tensors(), *split, workspace=ws, out=out, w_tiled=pw.tiled,
+                         norm_weight=gamma, eps=1e-5)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        run()                                # warm-up outside the capture (first-call setup)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            run()
+    torch.cuda.synchronize()
+    for i in (1, 2, 0, 1):
+        x_buf.copy_(xs[i])
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager = abi.fused_linear(xs[i], idx, *pw.tensors(), *split, w_tiled=pw.tiled, norm_weight=gamma, eps=1e-5)
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay with input {i} differs from the eager result"

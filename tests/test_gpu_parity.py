@@ -280,6 +280,52 @@ def test_config0_end_to_end(abi):
     assert rel < 0.2, rel
 
 
+# ------------------------------------------------------------------ the benchmark configurations at full size
+@pytest.mark.parametrize("cfg", ["c2", "c3", "c4"])
+def test_full_size_configs(abi, cfg):
+    """At the sizes the bench runs: weights bit-exact against the scalar oracle; a sample of token rows
+    (all of them for c2) against the oracle's GEMM; and two properties that need no oracle and cover every
+    tile -- permuting the token rows permutes the output rows bit for bit (a row's arithmetic does not
+    depend on where its tile sits), and doubling the activations (exact in bf16: codes unchanged, scale
+    exponents + 1) doubles every output exactly."""
+    m, n, k, kn, ks, ko = H.CONFIGS[cfg]
+    _say(cfg, "full size", m, n, k)
+    student = cfg == "c4"
+    x = H.make_activations(m, k, 1234 + int(cfg[1]), student_t=student)
+    w = H.make_weights(n, k, 2234 + int(cfg[1]))
+    idx = H.absmax_sort_index(x)
+    xd, wd, idd = x.to(DEV), w.to(DEV), idx.to(DEV)
+    bq = abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+    tiled = abi.weights_tileable(n, kn, ks, ko)
+    bt = (abi.tile_weights(*bq[:3]) + bq[3:]) if tiled else bq
+    d = abi.fused_linear(xd, idd, *bt, kn, ks, ko, w_tiled=tiled)
+    torch.cuda.synchronize()
+    H.assert_quant_equal(bq, sc.quantize_w(H.bf16_bits(w), idx.numpy(), kn, ks, ko), n, (kn, ks, ko), what=f"{cfg} w")
+
+    # sampled token rows against the oracle
+    rng = np.random.default_rng(7)
+    rows = np.arange(m) if m <= 64 else np.sort(rng.choice(m, 48, replace=False))
+    qx = mo.reorder_quantize_x(H.bf16_f32(x)[rows], idx.numpy(), kn, ks, ko)
+    qw = mo.reorder_quantize_w(H.bf16_f32(w), idx.numpy(), kn, ks, ko)
+    _check_gemm(d[torch.from_numpy(rows).to(DEV)], qx, qw, f"{cfg} sampled rows")
+    aq = abi.reorder_quantize_x(xd, idd, kn, ks, ko)
+    torch.cuda.synchronize()
+    want = sc.quantize_x(H.bf16_bits(x)[rows], idx.numpy(), kn, ks, ko)
+    for t, name in zip(aq[:3], ("qn", "qs", "qo")):
+        np.testing.assert_array_equal(t.cpu().numpy()[rows], want[name], err_msg=f"{cfg} {name}")
+
+    # token-row permutation
+    perm = torch.from_numpy(rng.permutation(m)).to(DEV)
+    d_perm = abi.fused_linear(xd[perm].contiguous(), idd, *bt, kn, ks, ko, w_tiled=tiled)
+    torch.cuda.synchronize()
+    assert torch.equal(d_perm, d[perm]), f"{cfg}: output rows do not follow a permutation of the token rows"
+
+    # activations x 2
+    d2 = abi.fused_linear((xd.float() * 2.0).to(torch.bfloat16), idd, *bt, kn, ks, ko, w_tiled=tiled)
+    torch.cuda.synchronize()
+    assert torch.equal(d2.float(), d.float() * 2.0), f"{cfg}: doubling the activations does not double the output"
+
+
 # ------------------------------------------------------------------ torch extension surface
 def test_extension_module_runs_the_reference_call_sequence(abi):
     import os

@@ -285,8 +285,8 @@ def test_config0_end_to_end(abi):
 def test_full_size_configs(abi, cfg):
     """At the sizes the bench runs: weights bit-exact against the scalar oracle; a sample of token rows
     (all of them for c2) against the oracle's GEMM; and two properties that need no oracle and cover every
-    tile -- permuting the token rows permutes the output rows bit for bit (a row's arithmetic does not
-    depend on where its tile sits), and doubling the activations (exact in bf16: codes unchanged, scale
+    tile -- repeated runs are bit-identical, permuting the token rows permutes the output rows bit for bit (a
+    row's arithmetic does not depend on where its tile sits), and doubling the activations (exact in bf16: codes unchanged, scale
     exponents + 1) doubles every output exactly."""
     m, n, k, kn, ks, ko = H.CONFIGS[cfg]
     _say(cfg, "full size", m, n, k)
@@ -313,6 +313,13 @@ def test_full_size_configs(abi, cfg):
     want = sc.quantize_x(H.bf16_bits(x)[rows], idx.numpy(), kn, ks, ko)
     for t, name in zip(aq[:3], ("qn", "qs", "qo")):
         np.testing.assert_array_equal(t.cpu().numpy()[rows], want[name], err_msg=f"{cfg} {name}")
+
+    # the same launch again, twice, with other work in between: bit-identical (no race in the copy pipeline)
+    for _ in range(2):
+        abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+        again = abi.fused_linear(xd, idd, *bt, kn, ks, ko, w_tiled=tiled)
+        torch.cuda.synchronize()
+        assert torch.equal(again, d), f"{cfg}: two runs of the same problem differ"
 
     # token-row permutation
     perm = torch.from_numpy(rng.permutation(m)).to(DEV)

@@ -5,7 +5,6 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from oracle import mx_oracle as mo
 
 # name -> (M, N, K, KN, KS, KO)
 CONFIGS = {
@@ -59,6 +58,7 @@ def random_index(k, seed):
 
 
 def gather_logical_scales(sf: torch.Tensor, rows: int, kseg: int) -> np.ndarray:
+    from oracle import mx_oracle as mo   # imported where it is used: bench.py takes its inputs from this module
     return mo.sf_gather(sf.detach().cpu().numpy(), rows, kseg)
 
 
@@ -66,6 +66,7 @@ def assert_quant_equal(got, want, rows, splits, what=""):
     """got: 6 device tensors; want: dict from the oracle (packed codes + laid-out
     scale buffers).  Codes bit-exact; scales compared at the logical entries only
     (rows past the end of the matrix are never written)."""
+    from oracle import mx_oracle as mo
     names = ("qn", "qs", "qo")
     for t, name in zip(got[:3], names):
         np.testing.assert_array_equal(t.cpu().numpy(), want[name], err_msg=f"{what} {name}")

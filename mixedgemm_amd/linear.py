@@ -58,10 +58,16 @@ class PackedWeights:
     reorder_index: torch.Tensor
     split: tuple[int, int, int]
     tiled: bool = False   # wn, ws, wo in the tile-major order of mg_tile_weights (same shapes)
+    features: int = 0     # output features that are real; 0 = every stored row (rows past it are zero padding)
+
+    @property
+    def rows(self) -> int:
+        """Stored weight rows (a multiple of 256 when the layer was padded for the whole-tile kernel)."""
+        return self.wn.shape[0] if self.split[0] else (self.ws.shape[0] if self.split[1] else self.wo.shape[0])
 
     @property
     def out_features(self) -> int:
-        return self.wn.shape[0] if self.split[0] else (self.ws.shape[0] if self.split[1] else self.wo.shape[0])
+        return self.features or self.rows
 
     @property
     def in_features(self) -> int:
@@ -75,12 +81,17 @@ class PackedWeights:
         """Quantizes bf16 weight[N, K] on its GPU (reorder_quantize_w of the reference,
         bindings.cpp:188-305); with `tile`, shapes that allow it are then put in tile-major order."""
         split = tuple(split) if split is not None else default_split(weight.shape[1])
+        n = weight.shape[0]
+        # the whole-tile kernel wants a multiple of 256 features: zero rows are cheap, the layer drops their outputs
+        if tile and n > 256 and n % 256 and abi.weights_tileable((n + 255) // 256 * 256, *split):
+            pad = torch.zeros(((n + 255) // 256 * 256 - n, weight.shape[1]), dtype=weight.dtype, device=weight.device)
+            weight = torch.cat([weight, pad])
         q = abi.reorder_quantize_w(weight, reorder_index, *split)
-        pw = cls(*q, reorder_index, split)
+        pw = cls(*q, reorder_index, split, False, n if weight.shape[0] != n else 0)
         return pw.tile() if tile and pw.tileable() else pw
 
     def tileable(self) -> bool:
-        return abi.weights_tileable(self.out_features, *self.split)
+        return abi.weights_tileable(self.rows, *self.split)
 
     def tile(self) -> "PackedWeights":
         """The same weights with the codes in tile-major order (GPU tensors).  The prefill kernel
@@ -90,10 +101,11 @@ class PackedWeights:
         if not self.tileable():
             raise ValueError("tile-major order needs N % 256 == 0 and three segments of at least 128 channels")
         wn, ws, wo = abi.tile_weights(self.wn, self.ws, self.wo)
-        return PackedWeights(wn, ws, wo, self.sfwn, self.sfws, self.sfwo, self.reorder_index, self.split, True)
+        return PackedWeights(wn, ws, wo, self.sfwn, self.sfws, self.sfwo, self.reorder_index, self.split, True, self.features)
 
     def to(self, device) -> "PackedWeights":
-        return PackedWeights(*(t.to(device) for t in self.tensors()), self.reorder_index.to(device), self.split, self.tiled)
+        return PackedWeights(*(t.to(device) for t in self.tensors()), self.reorder_index.to(device), self.split, self.tiled,
+                             self.features)
 
     # The file: MAGIC, u32 header length, u32 data offset, JSON header, then at the data offset
     # (a multiple of 256) the sections, each at a 256-byte aligned offset counted from there.
@@ -102,6 +114,7 @@ class PackedWeights:
         arrays = {name: t.detach().cpu().contiguous().numpy()
                   for name, t in zip(_SECTIONS, (*self.tensors(), self.reorder_index))}
         header = {"format": "mixedgemm-packed-weights", "version": 1, "out_features": self.out_features,
+                  "stored_rows": self.rows,
                   "in_features": self.in_features, "split": list(self.split),
                   "scale_layout": "128x4-interleaved-e8m0",
                   "code_layout": "tile-major-256x128" if self.tiled else "row-major", "sections": {}}
@@ -139,13 +152,17 @@ class PackedWeights:
         layout = header.get("code_layout", "row-major")
         if layout not in ("row-major", "tile-major-256x128"):
             raise ValueError(f"{path}: unknown code layout {layout}")
+        n_real = int(header.get("out_features", 0))
         pw = cls(*out, split, layout != "row-major")
+        pw.features = n_real if n_real != pw.rows else 0
         pw.validate()
         return pw
 
     def validate(self) -> None:
         kn, ks, ko = self.split
-        n = self.out_features
+        n = self.rows
+        if not 0 <= self.features <= n:
+            raise ValueError(f"{self.features} real features in {n} stored rows")
         want = {"wn": (n, kn // 2), "ws": (n, ks // 2), "wo": (n, ko // 2)}
         for name, shape in want.items():
             t = getattr(self, name)
@@ -298,7 +315,7 @@ class MixedLinear(torch.nn.Module):
 
     def packed(self) -> PackedWeights:
         return PackedWeights(self.wn, self.ws, self.wo, self.sfwn, self.sfws, self.sfwo, self.reorder_index, self.split,
-                             self.tiled)
+                             self.tiled, self.out_features if self.out_features != self.wn.shape[0] else 0)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         lead = x.shape[:-1]
@@ -312,6 +329,8 @@ class MixedLinear(torch.nn.Module):
         else:
             y = torch.ops.mixedgemm_amd.fused_linear(x2.contiguous(), self.reorder_index, self.wn, self.ws, self.wo,
                                                      self.sfwn, self.sfws, self.sfwo, *self.split, self.tiled)
+        if y.shape[1] != self.out_features:
+            y = y[:, :self.out_features]       # the padding rows of the weights
         if self.bias is not None:
             y = y + self.bias
         return y.reshape(*lead, self.out_features)

@@ -176,3 +176,25 @@ def test_layer_replayed_as_a_hip_graph(linear):
         eager = abi.fused_linear(xs[i], idx, *pw.tensors(), *split, w_tiled=pw.tiled, norm_weight=gamma, eps=1e-5)
         torch.cuda.synchronize()
         assert torch.equal(got, eager), f"replay with input {i} differs from the eager result"
+
+
+@pytest.mark.parametrize("m,n", [(300, 1000), (8, 300)])
+def test_layer_pads_odd_feature_counts_to_whole_tiles(linear, tmp_path, m, n):
+    """N that is not a multiple of 256: the packer appends zero rows so that the whole-tile kernel and
+    tile-major weights apply; the layer returns the real N columns, and the file keeps both counts."""
+    k = 4096
+    split = linear.default_split(k)
+    x = H.make_activations(m, k, 95)
+    w = H.make_weights(n, k, 96)
+    idx = H.absmax_sort_index(x)
+    pw = linear.PackedWeights.from_float(w.to(DEV), idx.to(DEV), split)
+    assert pw.out_features == n and pw.rows % 256 == 0 and pw.rows >= n and pw.tiled
+    path = str(tmp_path / "odd.mgw")
+    pw.save(path)
+    back = linear.PackedWeights.load(path, device=DEV)
+    assert back.out_features == n and back.rows == pw.rows and back.tiled
+    y = linear.MixedLinear(back)(x.to(DEV))
+    torch.cuda.synchronize()
+    assert y.shape == (m, n)
+    ref, slack = _oracle_linear(x, w, idx, split)
+    _close(y, ref, slack)

@@ -827,7 +827,8 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* 
 #pragma unroll 8
     for (int i = 0; i < 32; ++i) {
       const v4u v = *reinterpret_cast<const v4u*>(rd + i * 4 * kPitch);
-      if (i * 4 < rows_left) *reinterpret_cast<v4u*>(out + (size_t)i * 4 * N) = v;
+      // streaming store: the result is not read again here, and the XCD's L2 is better spent on the operands
+      if (i * 4 < rows_left) __builtin_nontemporal_store(v, reinterpret_cast<v4u*>(out + (size_t)i * 4 * N));
     }
   }
 }

@@ -183,6 +183,24 @@ def main():
             "row_major_runs_ms": [round(v, 5) for v in rm], "tile_major_runs_ms": [round(v, 5) for v in tl],
             "row_major_ms": round(rm_ms, 5), "row_major_tflops": round(flops / (rm_ms * 1e-3) / 1e12, 1),
             "tile_major_ms": round(tl_ms, 5), "tile_major_tflops": round(flops / (tl_ms * 1e-3) / 1e12, 1)}
+        # ------------------------------------------------------------ the same launch on all-zero operands: same
+        # instructions, addresses and bytes moved, but the multiplier arrays do not toggle -- separates what the
+        # kernel's structure costs from what the chip's power limit costs on real operand bits
+        zq = abi.reorder_quantize_x(torch.zeros_like(xd), idd, kn, ks, ko)
+        zw = abi.reorder_quantize_w(torch.zeros_like(wd), idd, kn, ks, ko)
+        zb = abi.tile_weights(*zw[:3])
+        zr, rr = [], []
+        for _ in range(5):
+            zr.append(graph_ms(lambda i: abi.matmul(zq[0], zb[0], zq[1], zb[1], zq[2], zb[2], zq[3], zw[3], zq[4], zw[4],
+                                                    zq[5], zw[5], out=d, w_tiled=True), 20, repeats=2))
+            rr.append(graph_ms(lambda i: abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4],
+                                                    aq[5], bq[5], out=d, w_tiled=True), 20, repeats=2))
+        z_ms, r_ms = sorted(zr)[2], sorted(rr)[2]
+        extra["gemm_c3_zero_operands"] = {
+            "note": "c3 GEMM launch with all-zero operand codes against the bench operands, medians of 5 interleaved runs of 20 launches",
+            "zero_ms": round(z_ms, 5), "zero_tflops": round(flops / (z_ms * 1e-3) / 1e12, 1),
+            "bench_operands_ms": round(r_ms, 5), "bench_operands_tflops": round(flops / (r_ms * 1e-3) / 1e12, 1)}
+        del zq, zw, zb
         # ------------------------------------------------------------ c1: reorder-quantize alone, HBM-bound
         m1, _, k1, kn1, ks1, ko1 = H.CONFIGS["c1"]
         nsets = 8                                    # 8 x 44 MB > 256 MB Infinity Cache

@@ -22,6 +22,8 @@
 // The result tile is transposed through LDS so that stores write 256 contiguous bytes per row.
 #include "mg_common.h"
 
+#include <type_traits>
+
 namespace mg {
 
 namespace {
@@ -824,12 +826,26 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* 
     const uint8_t* rd = stage + r * kPitch + cc * 16;
     uint16_t* out = d + (size_t)(c.m0 + c.wm * 128 + r) * N + c.n0 + c.wn * 128 + cc * 8;
     const int rows_left = m_store - (c.m0 + c.wm * 128 + r);   // token rows at or past m_store are not written
-#pragma unroll 8
-    for (int i = 0; i < 32; ++i) {
-      const v4u v = *reinterpret_cast<const v4u*>(rd + i * 4 * kPitch);
-      // streaming store: the result is not read again here, and the XCD's L2 is better spent on the operands
-      if (i * 4 < rows_left) __builtin_nontemporal_store(v, reinterpret_cast<v4u*>(out + (size_t)i * 4 * N));
-    }
+    // Eight reads in flight, then their eight stores: a read that is waited for before its own store costs a
+    // full LDS latency per row (which is what the compiler makes of the predicated form: it sinks each read
+    // into its store's block -- hence the separate path for tiles that are stored whole).  Streaming stores: the result is not read again here, and the XCD's L2 is
+    // better spent on the operands.
+    auto write_rows = [&](auto whole) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        v4u v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const v4u*>(rd + (b * 8 + j) * 4 * kPitch);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int i = b * 8 + j;
+          if (decltype(whole)::value || i * 4 < rows_left)
+            __builtin_nontemporal_store(v[j], reinterpret_cast<v4u*>(out + (size_t)i * 4 * N));
+        }
+      }
+    };
+    if (m_store - c.m0 >= kT) write_rows(std::true_type{});   // wave-uniform: every row of the tile is stored
+    else write_rows(std::false_type{});
   }
 }
 

@@ -90,8 +90,8 @@ int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, cons
  * The same GEMM with two things a caller may know about its buffers:
  *   a_rows -- an, as_, ao are readable for a_rows >= M token rows and sfan, sfas, sfao for
  *     mg_sf_bytes(a_rows, kseg, MG_OPERAND_A) bytes (what lies past row M is never used for a
- *     result).  With a_rows >= mg_padded_rows(M) a token count that is not a multiple of 256 runs on
- *     the whole-tile kernel like any other; a_rows == M is always valid.
+ *     result).  a_rows == M is always valid: the whole-tile kernel never reads past row a_rows - 1
+ *     (lanes of later rows read that row again) and never writes past row M - 1.
  *   flags  -- MG_FLAG_W_TILED: bn, bs, bo hold the codes in the tile-major order mg_tile_weights
  *     writes (same sizes; mg_weights_tileable(N, KN, KS, KO) must hold).  The prefill kernel's copies
  *     then read consecutive kilobytes, which is worth 10-15 % of its time.

@@ -651,7 +651,7 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO);
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
-                                 int M, int m_store, int N, int KN, int KS, int KO, bool w_tiled, void* d,
+                                 int M, int m_store, int a_rows, int N, int KN, int KS, int KO, bool w_tiled, void* d,
                                  hipStream_t stream);
 
 // Rough launch times in microseconds (measured on MI355X, K = 4096: a 128-wide stage takes ~1.05 us
@@ -678,25 +678,16 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
   if (w_tiled && !mixed_gemm_256_supported(256, N, KN, KS, KO)) return hipErrorInvalidValue;
   const int m_pad = (M + 255) / 256 * 256;
   const int steps = (KN + 127) / 128 + (KS + 127) / 128 + (KO + 127) / 128;
-  // whole 256-row tiles, the last one possibly reading rows past M (readable up to a_rows) and
-  // not writing them
-  if ((M == m_pad || a_rows >= m_pad) && mixed_gemm_256_supported(m_pad, N, KN, KS, KO) &&
+  // whole 256-row tiles; the last one does not write rows past M and reads no activation row past
+  // a_rows (lanes that would are pointed at the last readable row)
+  if (mixed_gemm_256_supported(m_pad, N, KN, KS, KO) &&
       (M >= 256 || pipelined_us(m_pad, N, steps) < skinny_us(M, N, steps)))
-    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_pad, M, N, KN, KS, KO,
-                                 w_tiled, d, stream);
+    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_pad, M, a_rows, N, KN, KS,
+                                 KO, w_tiled, d, stream);
   const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
   const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
   const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};
   if (M < 256 && KN + KS + KO > 0) return launch_skinny(d4, d6, d8, 0, M, N, w_tiled, static_cast<uint16_t*>(d), stream);
-  // ragged token count: whole 256-row tiles on the pipelined kernel (same pointers: rows are
-  // independent and a scale atom never spans a 256-row boundary), the last rows on the skinny one
-  const int m_main = M / 256 * 256;
-  if (m_main < M && mixed_gemm_256_supported(m_main, N, KN, KS, KO)) {
-    hipError_t e = launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_main, m_main, N, KN,
-                                         KS, KO, w_tiled, d, stream);
-    if (e != hipSuccess) return e;
-    return launch_skinny(d4, d6, d8, m_main, M, N, w_tiled, static_cast<uint16_t*>(d), stream);
-  }
   // the tiled kernel needs whole tiles and whole 128-wide K stages
   if (M % kTileM == 0 && N % kTileN == 0 && KN % kStageK == 0 && KS % kStageK == 0 && KO % kStageK == 0 &&
       KN + KS + KO > 0) {

@@ -130,40 +130,51 @@ __device__ __forceinline__ void copy16io(const uint8_t* base, unsigned voff, uns
                : : "v"(voff), "s"(base), "s"(lds_sreg), "n"(OFF - GOFF), "n"(GOFF) : "memory", "m0", "scc");
 }
 
+struct Ctx {
+  int n0, m0, lane, wave, wn, wm, total;
+  int rows_avail;      // activation rows that may be read from m0 on (codes and scales); 1 ... 256
+  unsigned lds_base;   // LDS byte offset of the dynamic shared memory
+};
+
 // Per-lane byte offsets of the copies, fixed for the whole kernel.
+// Token rows are clamped to the last readable row of the tile (rows_avail - 1): in the last, partial
+// token tile the lanes of rows past it copy that row again, into LDS rows of tokens that are never stored.
 struct LaneOffsets {
   unsigned w0, w1, w2;      // weights: 16 rows apart per lane quad, 64-byte rows of pitch ldb of segment 0 / 1 / 2; tile-major: 16 * lane
-  unsigned x4;              // E2M1 tokens: the same pattern with the pitch of segment 0
-  unsigned x8;              // E4M3 tokens: pitch lda of segment 2
-  unsigned x6a, x6b, x6c;   // E3M2 tokens: piece (64k + lane) % 6 of row 8 * ((64k + lane) / 6), k = 0, 1, 2
   unsigned s0, s1, s2;      // scale atoms: lanes 0-31 the first 128 rows, 32-63 the next 128
+  int lane, wave, last_row, prow;
 
-  __device__ __forceinline__ LaneOffsets(const Plan& p, int lane) {
+  __device__ __forceinline__ LaneOffsets(const Plan& p, const Ctx& cx) {
+    lane = cx.lane;
+    wave = cx.wave;
+    last_row = cx.rows_avail - 1;
     // quad k of a copy holds tile row j + 16 * (2 * (k % 8) + k / 8): rows 32t + i and 32t + i + 16 of a
     // fragment end up 512 B apart in their block, which the LDS reads conflict-free (64 B apart they collide)
     const unsigned k = lane >> 2, pr = 2 * (k & 7) + (k >> 3), c = lane & 3;
-    x4 = 16 * pr * (p.blk0 * 16) + c * 16;
-    w0 = p.w_tiled ? lane * 16 : x4;
+    prow = 16 * pr;
+    w0 = p.w_tiled ? lane * 16 : 16 * pr * (p.blk0 * 16) + c * 16;
     w1 = p.w_tiled ? lane * 16 : 16 * pr * (p.blk1 * 16) + c * 16;
     w2 = p.w_tiled ? lane * 16 : 16 * pr * (p.blk2 * 16) + c * 16;
-    x8 = 16 * pr * (p.blk2 * 32) + c * 16;
-    const unsigned lda6 = p.blk1 * 24, c0 = lane, c1 = 64 + lane, c2 = 128 + lane;
-    x6a = 8 * (c0 / 6) * lda6 + (c0 % 6) * 16;
-    x6b = 8 * (c1 / 6) * lda6 + (c1 % 6) * 16;
-    x6c = 8 * (c2 / 6) * lda6 + (c2 % 6) * 16;
-    const unsigned hi = lane >> 5, lo = (lane & 31) * 16;
+    // scale atoms: waves 1 and 3 copy the token atoms; the second one exists only past 128 readable rows
+    const unsigned hi = ((wave & 1) && cx.rows_avail <= 128) ? 0 : lane >> 5, lo = (lane & 31) * 16;
     s0 = hi * ((p.blk0 + 3) >> 2) * 512 + lo;
     s1 = hi * ((p.blk1 + 3) >> 2) * 512 + lo;
     s2 = hi * ((p.blk2 + 3) >> 2) * 512 + lo;
   }
+
+  // Byte offset, from the tile's first token row, that this lane reads in token copy kx of a stage of
+  // segment sg (row pitch lda).  E2M1: rows 4 * wave + kx + 16 * pr, 16-byte piece lane % 4; E4M3: rows
+  // 8 * (wave % 2) + kx + 16 * pr; E3M2: piece c % 6 of row 2 * wave + kx / 3 + 8 * (c / 6), c = 64 * (kx % 3) + lane.
+  __device__ __forceinline__ unsigned xoff(int sg, int kx, unsigned lda) const {
+    if (sg == 1) {
+      const int c = 64 * (kx % 3) + lane;
+      return (unsigned)min(8 * (c / 6) + 2 * wave + kx / 3, last_row) * lda + (c % 6) * 16;
+    }
+    const int first = sg == 0 ? 4 * wave : 8 * (wave & 1);
+    return (unsigned)min(prow + first + kx, last_row) * lda + (lane & 3) * 16;
+  }
 };
 
-struct Ctx {
-  int n0, m0, lane, wave, wn, wm, total;
-  unsigned lds_base;   // LDS byte offset of the dynamic shared memory
-};
-
-// Wave-uniform bases of the copies of global stage q (any segment).
 struct StageBases {
   const uint8_t *w, *x, *s;
   unsigned ldb, lda;
@@ -192,9 +203,8 @@ struct StageBases {
     } else {
       w = pb + (size_t)(c.n0 + c.wave * 4) * ldb + (size_t)ql * 64;
     }
-    // first token row of the wave: E2M1 4*wave (+kx), E3M2 2*wave (+kx/3), E4M3 8*(wave%2) (+kx) in K half wave/2
-    const unsigned xrow = sg == 0 ? c.wave * 4 : (sg == 1 ? c.wave * 2 : (c.wave & 1) * 8);
-    x = pa + (size_t)(c.m0 + xrow) * lda + (size_t)ql * rb + (sg == 2 ? (c.wave >> 1) * 64 : 0);
+    // the tile's first token row (the lanes' offsets carry the wave's rows); E4M3: K half wave / 2
+    x = pa + (size_t)c.m0 * lda + (size_t)ql * rb + (sg == 2 ? (c.wave >> 1) * 64 : 0);
     s = (c.wave & 1) == 0 ? psb + ((size_t)(c.n0 >> 7) * nst + ql) * 512 : psa + ((size_t)(c.m0 >> 7) * nst + ql) * 512;
   }
 };
@@ -220,13 +230,12 @@ struct GenericCopy {
     } else if constexpr (K < 12) {
       constexpr int kx = K - 4;
       if (b.seg == 0) {
-        if constexpr (kx < 4) copy16(b.x + (size_t)kx * b.lda, lo.x4, buf + kXOff + (wave * 4 + kx) * kBlk);
+        if constexpr (kx < 4) copy16(b.x, lo.xoff(0, kx, b.lda), buf + kXOff + (wave * 4 + kx) * kBlk);
       } else if (b.seg == 1) {
         if constexpr (kx < 6)
-          copy16(b.x + (size_t)(kx / 3) * b.lda, kx % 3 == 0 ? lo.x6a : (kx % 3 == 1 ? lo.x6b : lo.x6c),
-                 buf + kXOff + (wave * 2 + kx / 3) * kBlk6 + (kx % 3) * 1024);
+          copy16(b.x, lo.xoff(1, kx, b.lda), buf + kXOff + (wave * 2 + kx / 3) * kBlk6 + (kx % 3) * 1024);
       } else {
-        copy16(b.x + (size_t)kx * b.lda, lo.x8, buf + kXOff + (wave * 8 + kx) * kBlk);
+        copy16(b.x, lo.xoff(2, kx, b.lda), buf + kXOff + (wave * 8 + kx) * kBlk);
       }
     } else {
       copy16(b.s, pick3u(b.seg, lo.s0, lo.s1, lo.s2), buf + kSOff + (wave & 1) * 1024);
@@ -245,47 +254,49 @@ __device__ __forceinline__ void issue_range(const GenericCopy& cp, const LaneOff
 // Copies of stages inside one segment of format FMT: scalar bases advanced by one stage at a time,
 // per-lane offsets (one register per copy, the row step of the copy folded in) fixed.
 // WT: weights in tile-major order -- one per-lane offset (16 * lane) and immediates for all four
-// weight copies; vw[] then holds the E2M1 token offsets only.
+// weight copies; vw[] is then unused.
 template <int FMT, bool WT>
 struct LeanCopy {
   static constexpr int NX = Fmt<FMT>::x_copies;
-  // token copies: E2M1 shares the weight offsets (same pitch); E3M2 keeps one offset per third of a
-  // block and E4M3 one, the row step of copy k is added when it is issued (a scalar multiple of lda)
-  static constexpr int NV = FMT == kFmtE2M1 ? 0 : (FMT == kFmtE3M2 ? 3 : 1);
+  // token copies, rows clamped to the last readable one.  E2M1: one offset per copy.  E3M2: one per third
+  // of a block for its first row; bits 0-2 of vs say whether the second row is a row further on.  E4M3,
+  // of which there are few stages: the first copy's offset, and in its bits 0-2 how many of the seven
+  // row steps that follow stay inside the readable rows.  (All offsets are multiples of 16.)
+  static constexpr int NV = FMT == kFmtE4M3 ? 1 : (FMT == kFmtE3M2 ? 3 : 4);
   const uint8_t *w, *x, *s;        // bases of the stage being copied
   unsigned lds_w, lds_x, lds_s;    // LDS offsets of the wave's first weight / token block and scale atom pair in buffer 0
   unsigned lda;
-  unsigned vw[4], vx[NV > 0 ? NV : 1], vs, vlin;
+  unsigned vw[4], vx[NV], vs, vlin;
 
   __device__ __forceinline__ void init(const Plan& plan, int q, const LaneOffsets&, const Ctx& c) {
-    const LaneOffsets lo(plan, c.lane);   // recomputed here rather than kept in registers across the K loop
+    const LaneOffsets lo(plan, c);   // recomputed here rather than kept in registers across the K loop
     const StageBases b(plan, q, c);
     w = uni(b.w);
     x = uni(b.x);
     s = uni(b.s);
-    lda = __builtin_amdgcn_readfirstlane(b.lda);
     constexpr int sg = Fmt<FMT>::seg;
     const unsigned w_off = sg == 0 ? lo.w0 : (sg == 1 ? lo.w1 : lo.w2);
     vlin = c.lane * 16;
-    if constexpr (WT) {
-      if constexpr (FMT == kFmtE2M1) {
+    if constexpr (!WT) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) vw[k] = lo.x4 + k * b.lda;
+      for (int k = 0; k < 4; ++k) vw[k] = w_off + k * b.ldb;
+    }
+    lda = __builtin_amdgcn_readfirstlane(b.lda);
+    unsigned flags = 0;
+    if constexpr (FMT == kFmtE4M3) {
+      const int row0 = lo.prow + 8 * (c.wave & 1);
+      vx[0] = lo.xoff(2, 0, b.lda) | (unsigned)min(max(lo.last_row - row0, 0), 7);
+    } else if constexpr (FMT == kFmtE3M2) {
+#pragma unroll
+      for (int t = 0; t < 3; ++t) {
+        vx[t] = lo.xoff(1, t, b.lda);
+        flags |= (lo.xoff(1, 3 + t, b.lda) != vx[t] ? 1u : 0u) << t;
       }
     } else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) vw[k] = w_off + k * b.ldb;   // E2M1 tokens use them too: same pattern, same pitch
+      for (int k = 0; k < 4; ++k) vx[k] = lo.xoff(0, k, b.lda);
     }
-    if constexpr (FMT == kFmtE3M2) {
-      vx[0] = lo.x6a;
-      vx[1] = lo.x6b;
-      vx[2] = lo.x6c;
-    } else if constexpr (FMT == kFmtE4M3) {
-      vx[0] = lo.x8;
-    } else {
-      vx[0] = 0;
-    }
-    vs = sg == 0 ? lo.s0 : (sg == 1 ? lo.s1 : lo.s2);
+    vs = (sg == 0 ? lo.s0 : (sg == 1 ? lo.s1 : lo.s2)) | flags;
     lds_w = __builtin_amdgcn_readfirstlane(c.lds_base + kWOff + c.wave * 4 * kBlk);
     lds_x = __builtin_amdgcn_readfirstlane(c.lds_base + kXOff +
                                            c.wave * (FMT == kFmtE2M1 ? 4 * kBlk : (FMT == kFmtE3M2 ? 2 * kBlk6 : 8 * kBlk)));
@@ -308,12 +319,14 @@ struct LeanCopy {
       else copy16i<K * kBlk>(w, vw[K], lds_w + boff);
     } else if constexpr (K < 4 + NX) {
       constexpr int kx = K - 4;
-      if constexpr (FMT == kFmtE2M1) copy16i<kx * kBlk>(x, vw[kx], lds_x + boff);
-      else if constexpr (FMT == kFmtE3M2)
-        copy16i<(kx / 3) * kBlk6 + (kx % 3) * 1024>(x + (size_t)(kx / 3) * lda, vx[kx % 3], lds_x + boff);
-      else copy16i<kx * kBlk>(x + (size_t)kx * lda, vx[0], lds_x + boff);
+      if constexpr (FMT == kFmtE3M2)
+        copy16i<(kx / 3) * kBlk6 + (kx % 3) * 1024>(x, kx < 3 ? vx[kx] : vx[kx - 3] + ((vs >> (kx - 3)) & 1) * lda,
+                                                    lds_x + boff);
+      else if constexpr (FMT == kFmtE4M3)
+        copy16i<kx * kBlk>(x, (vx[0] & ~15u) + min((unsigned)kx, vx[0] & 7u) * lda, lds_x + boff);
+      else copy16i<kx * kBlk>(x, vx[kx], lds_x + boff);
     } else if constexpr (K == 12) {
-      copy16i<0>(s, vs, lds_s + boff);
+      copy16i<0>(s, FMT == kFmtE3M2 ? vs & ~15u : vs, lds_s + boff);
     }
   }
 };
@@ -661,7 +674,8 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
     Scales sc;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const unsigned n = c.n0 + c.wn * 128 + t * 32 + i, m = c.m0 + c.wm * 128 + t * 32 + i;
+      const unsigned n = c.n0 + c.wn * 128 + t * 32 + i;
+      const unsigned m = c.m0 + min(c.wm * 128 + t * 32 + i, c.rows_avail - 1);   // rows past the last readable one are never stored
       const v4i wv = *reinterpret_cast<const v4i*>(wbase + (size_t)n * wpitch + (size_t)max(kbc - wfirst, 0) * 16);
       const int sw = sfb[sf_offset(n, kbc, katoms)], sx = sfa[sf_offset(m, kbc, katoms)];
       f.w[t] = ok ? wv : z;
@@ -698,7 +712,7 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
 // REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
 template <bool REGULAR, bool REM, bool WT>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* __restrict__ d) {
+mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
   Plan plan;
   plan.a0 = uni(plan_arg.a0); plan.a1 = uni(plan_arg.a1); plan.a2 = uni(plan_arg.a2);
@@ -743,6 +757,7 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* 
   c.n0 = tile_n * kT;
   c.m0 = tile_m * kT;
   c.total = plan.total;
+  c.rows_avail = min(a_rows - c.m0, kT);
   c.lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
 
   v16f acc[4][4];
@@ -753,7 +768,7 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, uint16_t* 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
 
-  const LaneOffsets lo(plan, c.lane);
+  const LaneOffsets lo(plan, c);
   const WeightPtrs wp(lds, c);
 
   // prologue: stages 0 and 1 and the first copies of stage 2 in flight; wait for stage 0 only
@@ -862,12 +877,15 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
-                                 int M, int m_store, int N, int KN, int KS, int KO, bool w_tiled, void* d,
+                                 int M, int m_store, int a_rows, int N, int KN, int KS, int KO, bool w_tiled, void* d,
                                  hipStream_t stream) {
+  // M: whole tiles; rows [m_store, M) are computed but not stored; the activation buffers are read up to row
+  // a_rows - 1 only
+  if (m_store > M || m_store <= M - kT || a_rows < m_store) return hipErrorInvalidValue;
   // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
   const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
   const bool rem = (KN | KS | KO) % 128 != 0;
-  typedef void (*kernel_t)(Plan, int, int, int, uint16_t*);
+  typedef void (*kernel_t)(Plan, int, int, int, int, uint16_t*);
   // [tiled][regular][rem]
   const kernel_t kernels[2][2][2] = {
       {{mixed_gemm_256_kernel<false, false, false>, mixed_gemm_256_kernel<false, true, false>},
@@ -887,7 +905,7 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.w_tiled = w_tiled ? 1 : 0;
   const int tiles_n = N / kT, tiles_m = M / kT;
   hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store,
-                     static_cast<uint16_t*>(d));
+                     a_rows, static_cast<uint16_t*>(d));
   return hipGetLastError();
 }
 

@@ -474,6 +474,34 @@ def test_tiled_weights_give_the_same_result_bit_for_bit(abi, m, n, kn, ks, ko):
     _check_gemm(d3, qx, qw, "tiled, exact-size buffers")
 
 
+@pytest.mark.parametrize("m", [257, 258, 261, 263, 271, 272, 273, 384, 385, 511, 16, 129, 200])
+@pytest.mark.parametrize("n,kn,ks,ko", [(2048, 2560, 1408, 128), (512, 448, 416, 224)])
+def test_exact_size_activation_buffers_on_the_whole_tile_kernel(abi, m, n, kn, ks, ko):
+    """Activation buffers with no room past row M: the lanes of the last tile that would read past the last row
+    read that row again, and the result equals the padded-buffer one bit for bit.  Row counts around the lengths
+    of the runs of rows a lane copies (2, 4, 8), the 16-row copy blocks and the second scale atom (128 rows)."""
+    _say("exact-size", m, n, kn, ks, ko)
+    k = kn + ks + ko
+    x = H.make_activations(m, k, 71 + m, n_out=max(1, k // 32))
+    w = H.make_weights(n, k, 72 + n)
+    idx = H.absmax_sort_index(x)
+    xd, wd, idd = x.to(DEV), w.to(DEV), idx.to(DEV)
+    bq = abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+    bt = abi.tile_weights(*bq[:3])
+    aq = abi.reorder_quantize_x(xd, idd, kn, ks, ko)
+    tight = [t.clone() for t in aq]
+    assert all(t.untyped_storage().nbytes() == t.numel() for t in tight)
+    args = lambda a, b: (a[0], b[0], a[1], b[1], a[2], b[2], a[3], bq[3], a[4], bq[4], a[5], bq[5])
+    d_pad = abi.matmul(*args(aq, bq))
+    d_tight = abi.matmul(*args(tight, bq))
+    d_tight_t = abi.matmul(*args(tight, bt), w_tiled=True)
+    torch.cuda.synchronize()
+    qx, qw = _oracle_operands(x, w, idx, kn, ks, ko)
+    _check_gemm(d_tight, qx, qw, "exact-size buffers")
+    assert torch.equal(d_tight, d_tight_t)
+    assert torch.equal(d_pad, d_tight)
+
+
 def test_tiled_flag_is_refused_for_shapes_that_cannot_be_tiled(abi):
     from mixedgemm_amd.abi import MixedGemmError
     assert not abi.weights_tileable(256, 448, 416, 64) and not abi.weights_tileable(200, 128, 128, 128)

@@ -34,7 +34,7 @@ P46, P8 = 10100.0, 5000.0
 # counter's reading for `bench.py --calibrate-copy`; None where not measured.  The figures and the
 # commands are in profiles/.
 MEASURED_TRAFFIC = {
-    "gemm_c3": int((135876.8 * 1.99981 + 114688.0 * 1.0) * 1024),   # tile-major weights; L2 misses re-read operands ~7x; D written once
+    "gemm_c3": int((136029.3 * 1.99981 + 115702.9 * 1.0) * 1024),   # tile-major weights; L2 misses re-read operands ~7x; D written once
     "quant_c1": int((16455.2 * 1.99981 + 10883.8 * 1.0) * 1024),    # 44.8 MB against 44.2 MB algorithmic
     "decode_c2": int((18259.8 * 1.99981 + 224.0 * 1.0) * 1024),     # 37.6 MB against 31.4 MB algorithmic
     "calibrate_c1": int(((16413.1 + 1038.8 + 81.5) * 1.99981 + (2048.0 + 16.0 + 56.3) * 1.0) * 1024),   # three kernels

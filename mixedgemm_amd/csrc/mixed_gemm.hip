@@ -136,8 +136,8 @@ mixed_gemm_direct_kernel(const uint8_t* __restrict__ an, const uint8_t* __restri
 
 
 // ---------------------------------------------------------------------------
-// Skinny kernel: few tokens (decode, small batches, the ragged last rows of a
-// prefill), weights streamed once per 16 * G tokens (HBM- or L2-bound).
+// Skinny kernel: few tokens (decode, small batches), weights streamed once per
+// 16 * G tokens (HBM- or L2-bound).
 //
 // A workgroup of 4 waves owns 16 output features and G groups of 16 tokens; the K
 // steps (128 elements each, counted over the three segments) are dealt to the 4
@@ -162,7 +162,7 @@ __device__ __forceinline__ v4f decode_mfma(v8i wb, v8i xa, v4f acc, int sw, int 
 
 template <int G, int F>
 __global__ void __launch_bounds__(256)
-mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, int M, int N, int steps_per_wave,
+mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N, int steps_per_wave,
                          int w_tiled, uint16_t* __restrict__ d) {
   constexpr int S = G * F >= 8 ? 1 : 8 / (G * F);   // K steps a wave keeps in flight at once
   __shared__ float partial[4][F][G][16 * 16];
@@ -184,7 +184,7 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int m_base, i
     n_ok[f] = n[f] < N;
     nc[f] = min(n[f], N - 1);   // clamped rows: every load is in bounds and unconditional
   }
-  const int m0 = m_base + blockIdx.y * (G * 16) + i;      // this lane's token in group 0
+  const int m0 = blockIdx.y * (G * 16) + i;      // this lane's token in group 0
   const int total = s4.steps + s6.steps + s8.steps;
   v4f acc[F][G];
 #pragma unroll
@@ -329,9 +329,9 @@ static int skinny_feature_groups(int rows, int N) {
   return ceil_div(N, 32) * ceil_div(rows, 16 * g) >= 256 ? 2 : 1;
 }
 
-hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int m_base, int M, int N,
+hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int N,
                          bool w_tiled, uint16_t* d, hipStream_t stream) {
-  const int rows = M - m_base;
+  const int rows = M;
   const int steps_per_wave = (d4.steps + d6.steps + d8.steps + 3) / 4;
   const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
   // two feature groups per workgroup for 17-64 tokens: each activation fragment then serves 32 features
@@ -342,20 +342,20 @@ hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeS
   const int wt = w_tiled ? 1 : 0;
   switch (g) {
     case 1:
-      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<1, 2>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
-      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<1, 1>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<1, 2>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
+      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<1, 1>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
       break;
     case 2:
-      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<2, 2>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
-      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<2, 1>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<2, 2>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
+      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<2, 1>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
       break;
     case 4:
-      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<4, 2>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
-      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<4, 1>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<4, 2>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
+      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<4, 1>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
       break;
     default:
-      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<8, 2>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
-      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<8, 1>), grid, dim3(256), 0, stream, d4, d6, d8, m_base, M, N, steps_per_wave, wt, d);
+      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<8, 2>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
+      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<8, 1>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
       break;
   }
   return hipGetLastError();
@@ -687,7 +687,7 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
   const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
   const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
   const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};
-  if (M < 256 && KN + KS + KO > 0) return launch_skinny(d4, d6, d8, 0, M, N, w_tiled, static_cast<uint16_t*>(d), stream);
+  if (M < 256 && KN + KS + KO > 0) return launch_skinny(d4, d6, d8, M, N, w_tiled, static_cast<uint16_t*>(d), stream);
   // the tiled kernel needs whole tiles and whole 128-wide K stages
   if (M % kTileM == 0 && N % kTileN == 0 && KN % kStageK == 0 && KS % kStageK == 0 && KO % kStageK == 0 &&
       KN + KS + KO > 0) {

@@ -83,8 +83,8 @@ def test_c_host_program_reproduces_golden_vectors(tmp_path, path):
 
 
 def test_c_host_program_on_a_ragged_prefill_shape_with_tiled_weights(tmp_path):
-    """300 tokens x 512 features: whole tiles + skinny tail for the plain GEMM (exact-size buffers), whole
-    tiles with unstored rows and tile-major weights for the fused call."""
+    """300 tokens x 512 features from hipMalloc'ed exact-size buffers: the last token tile of the plain GEMM reads
+    no row past the 300th; the fused call runs the same tiles on its padded workspace, with tile-major weights."""
     m, n, split = 300, 512, (2560, 1408, 128)
     k = sum(split)
     x = H.make_activations(m, k, 501)

@@ -172,7 +172,7 @@ GEMM_SHAPES = [
     # skinny kernel with 2, 4 and 8 token groups: ragged M and N, partial K steps, an empty segment
     (17, 48, 256, 128, 128), (32, 200, 96, 160, 64), (50, 40, 2560, 1408, 128), (64, 64, 0, 4928, 448),
     (100, 256, 448, 224, 64), (128, 4096, 2560, 1408, 128), (255, 272, 128, 128, 128), (200, 1000, 640, 256, 256),
-    # ragged token count: whole 256-row tiles on the pipelined kernel + the last rows on the skinny one
+    # ragged token counts: the last 256-row tile stores only part of its rows
     (300, 512, 2560, 1408, 128), (257, 256, 384, 384, 384), (767, 256, 448, 416, 224),
     # 256 or more tokens with an empty segment: the LDS-tiled kernel
     (256, 256, 256, 0, 0), (384, 256, 0, 256, 128), (256, 512, 128, 0, 128),
@@ -249,7 +249,7 @@ def test_fused_linear_equals_quantize_then_gemm(abi, m, n, kn, ks, ko):
     aq = abi.reorder_quantize_x(xd, idd, kn, ks, ko)
     d1 = abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5])
     d2 = abi.fused_linear(xd, idd, bq[0], bq[1], bq[2], bq[3], bq[4], bq[5], kn, ks, ko)
-    # exact-size activation buffers (no room past M): whole tiles + the skinny kernel for the last rows
+    # exact-size activation buffers (no room past M): the last tile's lanes read no row past M
     tight = [t.clone() for t in aq]
     d3 = abi.matmul(tight[0], bq[0], tight[1], bq[1], tight[2], bq[2], tight[3], bq[3], tight[4], bq[4], tight[5], bq[5])
     torch.cuda.synchronize()
@@ -464,7 +464,7 @@ def test_tiled_weights_give_the_same_result_bit_for_bit(abi, m, n, kn, ks, ko):
     d0 = abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5])
     d1 = abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], w_tiled=True)
     d2 = abi.fused_linear(xd, idd, bt[0], bt[1], bt[2], bq[3], bq[4], bq[5], kn, ks, ko, w_tiled=True)
-    tight = [t.clone() for t in aq]    # exact-size activation buffers: whole tiles + skinny tail
+    tight = [t.clone() for t in aq]    # exact-size activation buffers
     d3 = abi.matmul(tight[0], bt[0], tight[1], bt[1], tight[2], bt[2], tight[3], bq[3], tight[4], bq[4], tight[5], bq[5],
                     w_tiled=True)
     torch.cuda.synchronize()

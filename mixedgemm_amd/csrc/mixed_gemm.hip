@@ -238,7 +238,9 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
         const int mc = min(m0 + gi * 16, M - 1);
         const uint8_t* xrow = pa + (size_t)mc * nblk * xbytes + q * 4 * xbytes;
         xa[k][gi] = *reinterpret_cast<const v4i*>(xrow + off_a);
-        xb[k][gi] = *reinterpret_cast<const v4i*>(xrow + off_b);
+        // E2M1 needs one piece only; a wave-uniform branch around the second load pays for G = 4 only (measured)
+        if (G != 4 || seg != 0) xb[k][gi] = *reinterpret_cast<const v4i*>(xrow + off_b);
+        else xb[k][gi] = v4i{0, 0, 0, 0};
         sx[k][gi] = psa[sf_offset(mc, 4 * q + gc, katoms)];
       }
     }

@@ -44,6 +44,9 @@ extern "C" {
  *   sfn/sfs/sfo    E8M0 scale bytes, one per 32 elements, in the 128-row x
  *                  4-block interleaved layout; mg_sf_bytes(M, Kseg, MG_OPERAND_A)
  *                  bytes each.  Entries of rows >= M are left untouched.
+ * Inputs are expected to be finite.  A 32-element block that holds an infinity or a NaN gets codes
+ * and a scale that are not specified (the reference's own arithmetic, log2 and a division by the
+ * scale, src/reorder.cu:172-197, is undefined there too); other blocks are not affected.
  */
 int mg_reorder_quantize_x(const void* x_bf16, const int16_t* idx, int M, int K, int KN, int KS, int KO,
                           uint8_t* qn, uint8_t* qs, uint8_t* qo,

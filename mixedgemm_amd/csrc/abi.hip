@@ -15,6 +15,7 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
                              int a_rows, int N, int KN, int KS, int KO, unsigned flags, void* d, hipStream_t stream);
 hipError_t launch_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, hipStream_t stream);
+bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO);
 size_t calibrate_workspace_bytes(int K);
 hipError_t launch_calibrate(const void* x, int rows, int K, int16_t* idx, void* workspace, hipStream_t stream);
 }  // namespace mg
@@ -99,7 +100,7 @@ int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, cons
 int mg_padded_rows(int M) { return M <= 0 ? 0 : (M + 255) / 256 * 256; }
 
 int mg_weights_tileable(int N, int KN, int KS, int KO) {
-  return N > 0 && N % 256 == 0 && KN >= 128 && KS >= 128 && KO >= 128 && (KN | KS | KO) % 32 == 0;
+  return N > 0 && N % 256 == 0 && mg::mixed_gemm_256_supported(256, N, KN, KS, KO);   // what the whole-tile kernel takes
 }
 
 int mg_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, void* stream) {

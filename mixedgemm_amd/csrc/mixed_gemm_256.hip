@@ -609,7 +609,13 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a
     stage_body<FMT, FR1, true, F1, F1, 1>(acc, a, a_next, sc, lcn, n1 > 1, lcn, n1 > 2, gc, lo, plan, q0 + ql, true, ring, wp,
                                           xp, xpn, c);
   } else if constexpr (REGULAR) {
-    // last segment: its own stages only, any n >= 1
+    // last segment: its own stages only, any n >= 1; first the stages whose copies all exist (no run-time
+    // switches in the body), then the last three
+    for (; ql + 3 < n; ++ql) {
+      stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, true, lc, true, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+                                              xp, c);
+      ring.rotate();
+    }
     for (; ql + 1 < n; ++ql) {
       stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, ql + 2 < n, lc, ql + 3 < n, gc, lo, plan, q0 + ql,
                                               true, ring, wp, xp, xp, c);
@@ -710,7 +716,9 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
 }
 
 // REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
-template <bool REGULAR, bool REM, bool WT>
+// SEGS: which activation segments the plan has, bit 0 E2M1 (always), bit 1 E3M2, bit 2 E4M3 -- the
+// prefetched fragments pass from a segment to the next one that exists, and their types are fixed here.
+template <bool REGULAR, bool REM, bool WT, int SEGS = 7>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
@@ -785,8 +793,9 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   }
   asm volatile("s_barrier" ::: "memory");
 
-  HalfFrags<kFmtE2M1> a4;
-  HalfFrags<kFmtE3M2> a6;
+  static_assert(SEGS == 7 || (REGULAR && !REM && (SEGS == 1 || SEGS == 3 || SEGS == 5)), "plans with an empty segment");
+  HalfFrags<kFmtE2M1> a4, none4;
+  HalfFrags<kFmtE3M2> a6, none6;
   HalfFrags<kFmtE4M3> a8, none;
   Scales sc;
   {
@@ -802,9 +811,19 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   LeanCopy<kFmtE4M3, WT> l8;
   LeanCopy<kFmtNone, WT> l0;
   if constexpr (REGULAR) l4.init(plan, 2, lo, c);
-  run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
-  run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
-  run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4 + n6, wp, lds, c);
+  if constexpr (SEGS == 7) {
+    run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
+    run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
+    run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4 + n6, wp, lds, c);
+  } else if constexpr (SEGS == 5) {
+    run_segment<kFmtE2M1, kFmtE4M3, kFmtE4M3, REGULAR>(acc, a4, sc, a8, l4, l8, gc, lo, plan, n4, n8, 0, wp, lds, c);
+    run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4, wp, lds, c);
+  } else if constexpr (SEGS == 3) {
+    run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
+    run_segment<kFmtE3M2, kFmtNone, kFmtE3M2, REGULAR>(acc, a6, sc, none6, l6, l0, gc, lo, plan, n6, 0, n4, wp, lds, c);
+  } else {
+    run_segment<kFmtE2M1, kFmtNone, kFmtE2M1, REGULAR>(acc, a4, sc, none4, l4, l0, gc, lo, plan, n4, 0, 0, wp, lds, c);
+  }
 
   if constexpr (REM) {
     __builtin_amdgcn_sched_barrier(0);
@@ -868,10 +887,18 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
 
 
 bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
+  if (M <= 0 || N <= 0 || KN < 0 || KS < 0 || KO < 0) return false;
+  if (M % kT != 0 || N % kT != 0 || KN % 32 != 0 || KS % 32 != 0 || KO % 32 != 0) return false;
   // all three segments with at least one whole 128-wide stage: the pipeline hands the prefetched
   // fragments from one segment's loop to the next, in the order E2M1 -> E3M2 -> E4M3
-  return M > 0 && N > 0 && M % kT == 0 && N % kT == 0 && KN % 32 == 0 && KS % 32 == 0 && KO % 32 == 0 && KN >= 128 &&
-         KS >= 128 && KO >= 128;
+  if (KN >= 128 && KS >= 128 && KO >= 128) return true;
+  // plans without E3M2 and / or E4M3 activations: whole stages only, and three of them in every segment
+  // that is followed by another (the variants with compiled-in segment-boundary copies)
+  if ((KN | KS | KO) % 128 != 0 || KN < 128) return false;
+  if (KS == 0 && KO == 0) return true;
+  if (KS == 0) return KN >= 384;
+  if (KO == 0) return KN >= 384;
+  return false;
 }
 
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
@@ -892,7 +919,13 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
        {mixed_gemm_256_kernel<true, false, false>, mixed_gemm_256_kernel<true, true, false>}},
       {{mixed_gemm_256_kernel<false, false, true>, mixed_gemm_256_kernel<false, true, true>},
        {mixed_gemm_256_kernel<true, false, true>, mixed_gemm_256_kernel<true, true, true>}}};
-  const kernel_t kernel = kernels[w_tiled][regular][rem];
+  // plans with an empty segment: [tiled][which]; which = 0: E2M1 only, 1: E2M1 + E3M2, 2: E2M1 + E4M3
+  const kernel_t partial[2][3] = {
+      {mixed_gemm_256_kernel<true, false, false, 1>, mixed_gemm_256_kernel<true, false, false, 3>,
+       mixed_gemm_256_kernel<true, false, false, 5>},
+      {mixed_gemm_256_kernel<true, false, true, 1>, mixed_gemm_256_kernel<true, false, true, 3>,
+       mixed_gemm_256_kernel<true, false, true, 5>}};
+  const kernel_t kernel = (KS > 0 && KO > 0) ? kernels[w_tiled][regular][rem] : partial[w_tiled][KS > 0 ? 1 : (KO > 0 ? 2 : 0)];
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kBuffers * kStage); e != hipSuccess) return e;
   Plan p;
   p.a0 = an; p.a1 = as_; p.a2 = ao;

@@ -174,7 +174,10 @@ GEMM_SHAPES = [
     (100, 256, 448, 224, 64), (128, 4096, 2560, 1408, 128), (255, 272, 128, 128, 128), (200, 1000, 640, 256, 256),
     # ragged token counts: the last 256-row tile stores only part of its rows
     (300, 512, 2560, 1408, 128), (257, 256, 384, 384, 384), (767, 256, 448, 416, 224),
-    # 256 or more tokens with an empty segment: the LDS-tiled kernel
+    # plans without E3M2 and / or E4M3 activations on the whole-tile kernel (fragments pass to the next segment that exists)
+    (256, 256, 512, 0, 0), (512, 512, 128, 0, 0), (300, 256, 384, 0, 128), (256, 512, 1024, 0, 256), (256, 256, 384, 256, 0),
+    (300, 512, 2560, 1536, 0), (1000, 256, 4096, 0, 0),
+    # 256 or more tokens with another empty segment: the LDS-tiled kernel
     (256, 256, 256, 0, 0), (384, 256, 0, 256, 128), (256, 512, 128, 0, 128),
 ]
 
@@ -442,6 +445,8 @@ TILED_SHAPES = [
     (256, 256, 128, 128, 128), (512, 512, 256, 384, 128), (256, 768, 2560, 1408, 128), (512, 256, 384, 512, 256),
     (300, 512, 2560, 1408, 128), (1000, 256, 384, 384, 384),
     (8, 512, 2560, 1408, 128), (20, 256, 128, 256, 128), (50, 768, 384, 128, 128), (130, 256, 2560, 896, 128),
+    # plans without E3M2 and / or E4M3 activations
+    (256, 256, 512, 0, 0), (300, 512, 384, 0, 128), (512, 256, 2560, 1536, 0), (40, 256, 1024, 0, 0),
     # segments that end 32, 64 or 96 elements past their last whole stage (kept row-major behind the tiled part)
     (256, 256, 448, 416, 224), (512, 512, 2240, 1248, 448), (300, 256, 160, 480, 352), (8, 256, 448, 416, 224),
     (40, 512, 2240, 1248, 448),

@@ -327,6 +327,22 @@ def main():
         extra["per_format_gemm"] = {"note": "c3's M, N and K with 3840 of the 4096 channels in one activation format; "
                                             "peak = the same blended nominal formula", "rows": per_format}
 
+        # ------------------------------------------------------------ plans without E3M2 and / or E4M3 activations
+        partial = []
+        for knf, ksf, kof in ((4096, 0, 0), (3968, 0, 128), (2560, 1536, 0)):
+            aqf = abi.reorder_quantize_x(xd, idd, knf, ksf, kof)
+            wqf = abi.reorder_quantize_w(wd, idd, knf, ksf, kof)
+            wtf = abi.tile_weights(*wqf[:3])
+            df = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            f_ms = graph_ms(lambda i: abi.matmul(aqf[0], wtf[0], aqf[1], wtf[1], aqf[2], wtf[2], aqf[3], wqf[3],
+                                                 aqf[4], wqf[4], aqf[5], wqf[5], out=df, w_tiled=True), 20)
+            pk = blended_peak(knf, ksf, kof)
+            tf = 2.0 * m * n * k / (f_ms * 1e-3) / 1e12
+            partial.append({"split": [knf, ksf, kof], "gemm_ms": round(f_ms, 5), "tflops": round(tf, 1),
+                            "peak": round(pk, 1), "frac": round(tf / pk, 4)})
+            del aqf, wqf, wtf, df
+        extra["plans_without_a_segment"] = {"note": "c3's M, N and K, tile-major weights, whole-tile kernel", "rows": partial}
+
         # ------------------------------------------------------------ what the matrix cores sustain on this box
         # register-resident scaled-MFMA loop on all CUs: with pseudo-random operand bits the chip hits its
         # power limit and clocks down, which bounds any GEMM on real data below the nominal peak

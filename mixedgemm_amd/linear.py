@@ -99,7 +99,7 @@ class PackedWeights:
         if self.tiled:
             return self
         if not self.tileable():
-            raise ValueError("tile-major order needs N % 256 == 0 and three segments of at least 128 channels")
+            raise ValueError("tile-major order needs N % 256 == 0 and a split the whole-tile kernel takes (abi.weights_tileable)")
         wn, ws, wo = abi.tile_weights(self.wn, self.ws, self.wo)
         return PackedWeights(wn, ws, wo, self.sfwn, self.sfws, self.sfwo, self.reorder_index, self.split, True, self.features)
 

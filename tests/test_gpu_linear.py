@@ -198,3 +198,22 @@ def test_layer_pads_odd_feature_counts_to_whole_tiles(linear, tmp_path, m, n):
     assert y.shape == (m, n)
     ref, slack = _oracle_linear(x, w, idx, split)
     _close(y, ref, slack)
+
+
+@pytest.mark.parametrize("split", [(512, 0, 0), (384, 0, 128), (384, 128, 0)])
+def test_layer_with_a_plan_that_has_no_e3m2_or_e4m3_segment(linear, tmp_path, split):
+    """All-MXFP4 activations, MXFP4 + MXFP8 outliers, MXFP4 + MXFP6: packed tile-major, saved, loaded, run."""
+    m, n, k = 300, 512, sum(split)
+    x = H.make_activations(m, k, 97, n_out=8)
+    w = H.make_weights(n, k, 98)
+    idx = H.absmax_sort_index(x)
+    pw = linear.PackedWeights.from_float(w.to(DEV), idx.to(DEV), split)
+    assert pw.tiled
+    path = str(tmp_path / "partial.mgw")
+    pw.save(path)
+    back = linear.PackedWeights.load(path, device=DEV)
+    assert back.split == tuple(split) and back.tiled
+    y = linear.MixedLinear(back)(x.to(DEV))
+    torch.cuda.synchronize()
+    ref, slack = _oracle_linear(x, w, idx, split)
+    _close(y, ref, slack)

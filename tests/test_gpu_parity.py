@@ -507,6 +507,51 @@ def test_exact_size_activation_buffers_on_the_whole_tile_kernel(abi, m, n, kn, k
     assert torch.equal(d_pad, d_tight)
 
 
+def _seeded_shapes(count, seed):
+    """Shapes drawn across the dispatcher's cases: token counts on both sides of 256 and of whole tiles, feature
+    counts with and without whole 256-feature tiles, segments of 0 or 32..1024 channels in steps of 32."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        m = int(rng.choice([rng.integers(1, 40), rng.integers(40, 256), rng.integers(256, 700)]))
+        n = int(rng.choice([256 * rng.integers(1, 3), 16 * rng.integers(1, 40), rng.integers(1, 300)]))
+        seg = lambda: int(rng.choice([0, 32 * rng.integers(1, 8), 128 * rng.integers(1, 8)]))
+        kn, ks, ko = seg(), seg(), seg()
+        if kn + ks + ko == 0:
+            continue
+        out.append((m, n, kn, ks, ko))
+    return out
+
+
+@pytest.mark.parametrize("m,n,kn,ks,ko", _seeded_shapes(48, 20250))
+def test_seeded_shape_sweep_against_the_oracle(abi, m, n, kn, ks, ko):
+    """Whatever kernel the dispatcher picks, quantize + GEMM (padded and exact-size activation buffers, row-major
+    and, where the shape allows it, tile-major weights) agree with the oracle and with each other."""
+    _say("sweep", m, n, kn, ks, ko)
+    k = kn + ks + ko
+    x = H.make_activations(m, k, 7 + m + k, n_out=max(1, k // 32))
+    w = H.make_weights(n, k, 9 + n + k)
+    idx = H.random_index(k, m + n)
+    xd, wd, idd = x.to(DEV), w.to(DEV), idx.to(DEV)
+    bq = abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+    aq = abi.reorder_quantize_x(xd, idd, kn, ks, ko)
+    tight = [t.clone() for t in aq]
+    args = lambda a, b: (a[0], b[0], a[1], b[1], a[2], b[2], a[3], bq[3], a[4], bq[4], a[5], bq[5])
+    d_pad = abi.matmul(*args(aq, bq))
+    d_tight = abi.matmul(*args(tight, bq))
+    d_fused = abi.fused_linear(xd, idd, *bq, kn, ks, ko)
+    torch.cuda.synchronize()
+    qx, qw = _oracle_operands(x, w, idx, kn, ks, ko)
+    _check_gemm(d_pad, qx, qw, "padded buffers")
+    _check_gemm(d_tight, qx, qw, "exact-size buffers")
+    assert torch.equal(d_pad, d_fused)
+    if abi.weights_tileable(n, kn, ks, ko):
+        bt = abi.tile_weights(*bq[:3])
+        d_t = abi.matmul(*args(tight, bt), w_tiled=True)
+        torch.cuda.synchronize()
+        _check_gemm(d_t, qx, qw, "tile-major weights")
+
+
 def test_tiled_flag_is_refused_for_shapes_that_cannot_be_tiled(abi):
     from mixedgemm_amd.abi import MixedGemmError
     assert not abi.weights_tileable(256, 448, 416, 64) and not abi.weights_tileable(200, 128, 128, 128)

@@ -523,7 +523,22 @@ def _seeded_shapes(count, seed):
     return out
 
 
-@pytest.mark.parametrize("m,n,kn,ks,ko", _seeded_shapes(48, 20250))
+def _seeded_tile_shapes(count, seed):
+    """Shapes the whole-tile kernel takes: ragged token counts, segments of whole stages or with 32, 64, 96 channels
+    past them, with and without three stages before a boundary, plans without E3M2 and / or E4M3."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        m = int(rng.integers(1, 600))
+        n = 256 * int(rng.integers(1, 3))
+        kn = int(rng.choice([128 * rng.integers(1, 9), 128 + 32 * rng.integers(0, 30)]))
+        ks = int(rng.choice([0, 128 * rng.integers(1, 7), 128 + 32 * rng.integers(0, 20)]))
+        ko = int(rng.choice([0, 128 * rng.integers(1, 4), 128 + 32 * rng.integers(0, 8)]))
+        out.append((m, n, kn, ks, ko))
+    return out
+
+
+@pytest.mark.parametrize("m,n,kn,ks,ko", _seeded_shapes(48, 20250) + _seeded_tile_shapes(40, 777))
 def test_seeded_shape_sweep_against_the_oracle(abi, m, n, kn, ks, ko):
     """Whatever kernel the dispatcher picks, quantize + GEMM (padded and exact-size activation buffers, row-major
     and, where the shape allows it, tile-major weights) agree with the oracle and with each other."""

@@ -113,7 +113,7 @@ int mg_mixed_gemm_ex(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, c
  * it; the 1-3 blocks of 32 a segment may have past its last whole stage follow as row-major rows.
  * N a multiple of 256, kseg a multiple of 32.  Done once per layer, offline. */
 int mg_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, void* stream);
-/* 1 when weights of this shape can be tiled (the shapes the whole-tile kernel takes): N a multiple of
+/* 1 when weights of this shape can be tiled (the shapes the whole-tile kernel takes, whole tiles only): N a multiple of
  * 256 and either every segment a multiple of 32 and at least 128 wide, or KS and / or KO zero with the
  * other segments multiples of 128 (KN >= 384 when a segment follows it). */
 int mg_weights_tileable(int N, int KN, int KS, int KO);

@@ -661,7 +661,7 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
 // round of 256 tiles; 0.19-0.25 ns per 16 tokens x 16 features x 128 K on the skinny kernel), only to
 // choose between the two for fewer than 256 tokens.
 static double pipelined_us(int m_pad, int N, int stages) {
-  const int tiles = (m_pad / 256) * (N / 256);
+  const int tiles = (m_pad / 256) * ((N + 255) / 256);
   return (double)((tiles + 255) / 256) * (stages * (tiles <= 128 ? 0.7 : 1.05) + 8.0);
 }
 static double skinny_us(int rows, int N, int steps) {
@@ -677,7 +677,7 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
   if (M == 0 || N == 0) return hipSuccess;
   const bool w_tiled = (flags & 1u) != 0;   // MG_FLAG_W_TILED
   // tile-major weights exist only for shapes the 256x256 kernel takes
-  if (w_tiled && !mixed_gemm_256_supported(256, N, KN, KS, KO)) return hipErrorInvalidValue;
+  if (w_tiled && (N % 256 != 0 || !mixed_gemm_256_supported(256, N, KN, KS, KO))) return hipErrorInvalidValue;
   const int m_pad = (M + 255) / 256 * 256;
   const int steps = (KN + 127) / 128 + (KS + 127) / 128 + (KO + 127) / 128;
   // whole 256-row tiles; the last one does not write rows past M and reads no activation row past

@@ -133,6 +133,7 @@ __device__ __forceinline__ void copy16io(const uint8_t* base, unsigned voff, uns
 struct Ctx {
   int n0, m0, lane, wave, wn, wm, total;
   int rows_avail;      // activation rows that may be read from m0 on (codes and scales); 1 ... 256
+  int cols_avail;      // features of the tile that exist (weight rows and scales that may be read from n0 on); 1 ... 256
   unsigned lds_base;   // LDS byte offset of the dynamic shared memory
 };
 
@@ -140,26 +141,30 @@ struct Ctx {
 // Token rows are clamped to the last readable row of the tile (rows_avail - 1): in the last, partial
 // token tile the lanes of rows past it copy that row again, into LDS rows of tokens that are never stored.
 struct LaneOffsets {
-  unsigned w0, w1, w2;      // weights: 16 rows apart per lane quad, 64-byte rows of pitch ldb of segment 0 / 1 / 2; tile-major: 16 * lane
   unsigned s0, s1, s2;      // scale atoms: lanes 0-31 the first 128 rows, 32-63 the next 128
-  int lane, wave, last_row, prow;
+  int lane, wave, last_row, last_col, prow;
 
   __device__ __forceinline__ LaneOffsets(const Plan& p, const Ctx& cx) {
     lane = cx.lane;
     wave = cx.wave;
     last_row = cx.rows_avail - 1;
+    last_col = cx.cols_avail - 1;
     // quad k of a copy holds tile row j + 16 * (2 * (k % 8) + k / 8): rows 32t + i and 32t + i + 16 of a
     // fragment end up 512 B apart in their block, which the LDS reads conflict-free (64 B apart they collide)
-    const unsigned k = lane >> 2, pr = 2 * (k & 7) + (k >> 3), c = lane & 3;
+    const unsigned k = lane >> 2, pr = 2 * (k & 7) + (k >> 3);
     prow = 16 * pr;
-    w0 = p.w_tiled ? lane * 16 : 16 * pr * (p.blk0 * 16) + c * 16;
-    w1 = p.w_tiled ? lane * 16 : 16 * pr * (p.blk1 * 16) + c * 16;
-    w2 = p.w_tiled ? lane * 16 : 16 * pr * (p.blk2 * 16) + c * 16;
-    // scale atoms: waves 1 and 3 copy the token atoms; the second one exists only past 128 readable rows
-    const unsigned hi = ((wave & 1) && cx.rows_avail <= 128) ? 0 : lane >> 5, lo = (lane & 31) * 16;
+    // scale atoms: waves 0 and 2 copy the feature atoms, 1 and 3 the token atoms; the second atom of a
+    // tile exists only past 128 features / readable token rows
+    const unsigned hi = ((wave & 1) ? cx.rows_avail : cx.cols_avail) <= 128 ? 0 : lane >> 5, lo = (lane & 31) * 16;
     s0 = hi * ((p.blk0 + 3) >> 2) * 512 + lo;
     s1 = hi * ((p.blk1 + 3) >> 2) * 512 + lo;
     s2 = hi * ((p.blk2 + 3) >> 2) * 512 + lo;
+  }
+
+  // Byte offset, from the tile's first weight row, that this lane reads in weight copy k of a stage (row-major
+  // weights, row pitch ldb): 64 bytes of row 4 * wave + k + 16 * pr, clamped to the last feature that exists.
+  __device__ __forceinline__ unsigned woff(int k, unsigned ldb) const {
+    return (unsigned)min(prow + 4 * wave + k, last_col) * ldb + (lane & 3) * 16;
   }
 
   // Byte offset, from the tile's first token row, that this lane reads in token copy kx of a stage of
@@ -179,8 +184,9 @@ struct StageBases {
   const uint8_t *w, *x, *s;
   unsigned ldb, lda;
   int seg;   // -1: no such stage
+  bool tiled;   // tile-major weights
 
-  __device__ __forceinline__ StageBases() : w(nullptr), x(nullptr), s(nullptr), ldb(0), lda(0), seg(-1) {}
+  __device__ __forceinline__ StageBases() : w(nullptr), x(nullptr), s(nullptr), ldb(0), lda(0), seg(-1), tiled(false) {}
 
   __device__ __forceinline__ StageBases(const Plan& plan, int q, const Ctx& c) {
     int ql;
@@ -195,13 +201,14 @@ struct StageBases {
     const unsigned rb = sg == 0 ? 64 : (sg == 1 ? 96 : 128);
     ldb = blk * 16;
     lda = blk * (rb >> 2);
+    tiled = plan.w_tiled != 0;
     if (plan.w_tiled) {
       // 16 KB per (feature tile, stage), 1 KB per copy block: the wave's 4 blocks are consecutive
       const unsigned nstg = (unsigned)pick3(sg, (uint64_t)plan.st0, (uint64_t)plan.st1, (uint64_t)plan.st2);
       w = pb + (((size_t)(c.n0 >> 8) * nstg + ql) * 16 + c.wave * 4) * 1024;
       ldb = 1024;
     } else {
-      w = pb + (size_t)(c.n0 + c.wave * 4) * ldb + (size_t)ql * 64;
+      w = pb + (size_t)c.n0 * ldb + (size_t)ql * 64;   // the lanes' offsets carry the wave's rows
     }
     // the tile's first token row (the lanes' offsets carry the wave's rows); E4M3: K half wave / 2
     x = pa + (size_t)c.m0 * lda + (size_t)ql * rb + (sg == 2 ? (c.wave >> 1) * 64 : 0);
@@ -226,7 +233,8 @@ struct GenericCopy {
   __device__ __forceinline__ void issue(const LaneOffsets& lo, int wave) const {
     if (b.seg < 0) return;
     if constexpr (K < 4) {
-      copy16(b.w + (size_t)K * b.ldb, pick3u(b.seg, lo.w0, lo.w1, lo.w2), buf + kWOff + (wave * 4 + K) * kBlk);
+      if (b.tiled) copy16(b.w + (size_t)K * 1024, lo.lane * 16, buf + kWOff + (wave * 4 + K) * kBlk);
+      else copy16(b.w, lo.woff(K, b.ldb), buf + kWOff + (wave * 4 + K) * kBlk);
     } else if constexpr (K < 12) {
       constexpr int kx = K - 4;
       if (b.seg == 0) {
@@ -275,11 +283,10 @@ struct LeanCopy {
     x = uni(b.x);
     s = uni(b.s);
     constexpr int sg = Fmt<FMT>::seg;
-    const unsigned w_off = sg == 0 ? lo.w0 : (sg == 1 ? lo.w1 : lo.w2);
     vlin = c.lane * 16;
     if constexpr (!WT) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) vw[k] = w_off + k * b.ldb;
+      for (int k = 0; k < 4; ++k) vw[k] = lo.woff(k, b.ldb);
     }
     lda = __builtin_amdgcn_readfirstlane(b.lda);
     unsigned flags = 0;
@@ -680,7 +687,7 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
     Scales sc;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const unsigned n = c.n0 + c.wn * 128 + t * 32 + i;
+      const unsigned n = c.n0 + min(c.wn * 128 + t * 32 + i, c.cols_avail - 1);   // features past the last one are never stored
       const unsigned m = c.m0 + min(c.wm * 128 + t * 32 + i, c.rows_avail - 1);   // rows past the last readable one are never stored
       const v4i wv = *reinterpret_cast<const v4i*>(wbase + (size_t)n * wpitch + (size_t)max(kbc - wfirst, 0) * 16);
       const int sw = sfb[sf_offset(n, kbc, katoms)], sx = sfa[sf_offset(m, kbc, katoms)];
@@ -766,6 +773,7 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   c.m0 = tile_m * kT;
   c.total = plan.total;
   c.rows_avail = min(a_rows - c.m0, kT);
+  c.cols_avail = min(N - c.n0, kT);
   c.lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
 
   v16f acc[4][4];
@@ -859,7 +867,8 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
     const int r = c.lane >> 4, cc = c.lane & 15;
     const uint8_t* rd = stage + r * kPitch + cc * 16;
     uint16_t* out = d + (size_t)(c.m0 + c.wm * 128 + r) * N + c.n0 + c.wn * 128 + cc * 8;
-    const int rows_left = m_store - (c.m0 + c.wm * 128 + r);   // token rows at or past m_store are not written
+    // token rows at or past m_store are not written, nor the 8-feature pieces past the layer's last feature
+    const int rows_left = (c.wn * 128 + cc * 8 < c.cols_avail) ? m_store - (c.m0 + c.wm * 128 + r) : 0;
     // Eight reads in flight, then their eight stores: a read that is waited for before its own store costs a
     // full LDS latency per row (which is what the compiler makes of the predicated form: it sinks each read
     // into its store's block -- hence the separate path for tiles that are stored whole).  Streaming stores: the result is not read again here, and the XCD's L2 is
@@ -878,7 +887,7 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
         }
       }
     };
-    if (m_store - c.m0 >= kT) write_rows(std::true_type{});   // wave-uniform: every row of the tile is stored
+    if (m_store - c.m0 >= kT && c.cols_avail == kT) write_rows(std::true_type{});   // wave-uniform: the whole tile is stored
     else write_rows(std::false_type{});
   }
 }
@@ -888,7 +897,8 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
 
 bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
   if (M <= 0 || N <= 0 || KN < 0 || KS < 0 || KO < 0) return false;
-  if (M % kT != 0 || N % kT != 0 || KN % 32 != 0 || KS % 32 != 0 || KO % 32 != 0) return false;
+  // N: whole 8-feature store pieces (tile-major weights need whole tiles: mg_weights_tileable)
+  if (M % kT != 0 || N % 8 != 0 || KN % 32 != 0 || KS % 32 != 0 || KO % 32 != 0) return false;
   // all three segments with at least one whole 128-wide stage: the pipeline hands the prefetched
   // fragments from one segment's loop to the next, in the order E2M1 -> E3M2 -> E4M3
   if (KN >= 128 && KS >= 128 && KO >= 128) return true;
@@ -936,7 +946,8 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.blk0 = KN / 32; p.blk1 = KS / 32; p.blk2 = KO / 32;
   p.total = p.st0 + p.st1 + p.st2;
   p.w_tiled = w_tiled ? 1 : 0;
-  const int tiles_n = N / kT, tiles_m = M / kT;
+  if (w_tiled && N % kT != 0) return hipErrorInvalidValue;
+  const int tiles_n = (N + kT - 1) / kT, tiles_m = M / kT;
   hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store,
                      a_rows, static_cast<uint16_t*>(d));
   return hipGetLastError();

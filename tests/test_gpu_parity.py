@@ -177,6 +177,10 @@ GEMM_SHAPES = [
     # plans without E3M2 and / or E4M3 activations on the whole-tile kernel (fragments pass to the next segment that exists)
     (256, 256, 512, 0, 0), (512, 512, 128, 0, 0), (300, 256, 384, 0, 128), (256, 512, 1024, 0, 256), (256, 256, 384, 256, 0),
     (300, 512, 2560, 1536, 0), (1000, 256, 4096, 0, 0),
+    # feature counts that are not whole 256-feature tiles (multiples of 8): the last tile's lanes read the last
+    # weight row again and store only the pieces that exist
+    (300, 1000, 2560, 1408, 128), (256, 264, 384, 384, 384), (512, 136, 448, 416, 224), (700, 8, 128, 128, 128),
+    (256, 392, 512, 0, 0), (384, 648, 384, 0, 128),
     # 256 or more tokens with another empty segment: the LDS-tiled kernel
     (256, 256, 256, 0, 0), (384, 256, 0, 256, 128), (256, 512, 128, 0, 128),
 ]

@@ -31,14 +31,56 @@ P46, P8 = 10100.0, 5000.0
 
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the same
-# counter's reading for `bench.py --calibrate-copy`; None where not measured.  The figures and the
-# commands are in profiles/.
+# counter's reading for `bench.py --calibrate-copy`.  These are figures of an earlier profiling run, not of
+# this one: each entry names the summary under profiles/ it comes from and the SHA-256 (first 16 hex digits)
+# of the kernel source it was taken with; when the source has changed since, the JSON carries null and says so.
+PROFILE = "profiles/hbm_traffic_fetch_write_size.txt"
 MEASURED_TRAFFIC = {
-    "gemm_c3": int((136029.3 * 1.99981 + 115702.9 * 1.0) * 1024),   # tile-major weights; L2 misses re-read operands ~7x; D written once
-    "quant_c1": int((16455.2 * 1.99981 + 10883.8 * 1.0) * 1024),    # 44.8 MB against 44.2 MB algorithmic
-    "decode_c2": int((18259.8 * 1.99981 + 224.0 * 1.0) * 1024),     # 37.6 MB against 31.4 MB algorithmic
-    "calibrate_c1": int(((16413.1 + 1038.8 + 81.5) * 1.99981 + (2048.0 + 16.0 + 56.3) * 1.0) * 1024),   # three kernels
+    "gemm_c3": {"bytes": int((136029.3 * 1.99981 + 115702.9 * 1.0) * 1024),      # 397 MB against 159 MB algorithmic: operands re-read 2.5x past L2
+                "source": "mixedgemm_amd/csrc/mixed_gemm_256.hip", "sha": "TBD"},
+    "quant_c1": {"bytes": int((16455.2 * 1.99981 + 10883.8 * 1.0) * 1024),       # 44.8 MB against 44.2 MB algorithmic
+                 "source": "mixedgemm_amd/csrc/reorder_quant.hip", "sha": "TBD"},
+    "decode_c2": {"bytes": int((18259.8 * 1.99981 + 224.0 * 1.0) * 1024),        # 37.6 MB against 31.4 MB algorithmic
+                  "source": "mixedgemm_amd/csrc/mixed_gemm.hip", "sha": "TBD"},
+    "calibrate_c1": {"bytes": int(((16413.1 + 1038.8 + 81.5) * 1.99981 + (2048.0 + 16.0 + 56.3) * 1.0) * 1024),   # three kernels
+                     "source": "mixedgemm_amd/csrc/calibrate.hip", "sha": "TBD"},
 }
+
+
+def source_sha(rel):
+    import hashlib
+    with open(os.path.join(ROOT, rel), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def traffic(key):
+    """(bytes or None, provenance string) of a kernel's profiled HBM traffic."""
+    e = MEASURED_TRAFFIC[key]
+    now = source_sha(e["source"])
+    if now != e["sha"]:
+        return None, f"not re-profiled since {e['source']} changed (figure in {PROFILE} was taken at source sha256 {e['sha']}, now {now})"
+    return e["bytes"], f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE figure from {PROFILE}, taken at {e['source']} sha256 {e['sha']} (unchanged since); not measured by this run"
+
+
+def bench_lib():
+    """The measurement kernels (libmixedgemm_bench.so): MFMA register loop, streaming copy, empty launch."""
+    import ctypes
+    path = os.path.join(ROOT, "mixedgemm_amd", "lib", "libmixedgemm_bench.so")
+    L = ctypes.CDLL(path)
+    p, i, z = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    L.mgb_measure_mfma_ceiling.restype = i
+    L.mgb_measure_mfma_ceiling.argtypes = [i, i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    L.mgb_stream.restype, L.mgb_stream.argtypes = i, [p, z, p, z, i, p]
+    L.mgb_empty_launch.restype, L.mgb_empty_launch.argtypes = i, [i, i, p]
+    return L
+
+
+def measure_mfma_ceiling(L, random_operands, iters=4000):
+    import ctypes
+    tf, ghz = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    rc = L.mgb_measure_mfma_ceiling(int(bool(random_operands)), iters, ctypes.byref(tf), ctypes.byref(ghz))
+    assert rc == 0, f"mgb_measure_mfma_ceiling: {rc}"
+    return tf.value, ghz.value
 
 
 def blended_peak(kn, ks, ko):
@@ -93,7 +135,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -136,40 +178,88 @@ def main():
     bt = abi.tile_weights(*bq[:3])
     aq = abi.alloc_quant_outputs(m, kn, ks, ko, abi.MG_OPERAND_A, dev)
     d = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(abi.fused_workspace_bytes(m, kn, ks, ko), dtype=torch.uint8, device=dev)
     torch.cuda.synchronize()
 
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    # The step: ONE call of mg_fused_linear_ex (reorder-quantize into the preallocated workspace, then the
+    # GEMM, on torch's current stream), arguments converted once.
+    import ctypes
+    L = abi.lib()
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    fused_args = (vp(xd), vp(idd), vp(bt[0]), vp(bt[1]), vp(bt[2]), vp(bq[3]), vp(bq[4]), vp(bq[5]), m, n, kn, ks, ko,
+                  abi.MG_FLAG_W_TILED, vp(d), vp(ws), ctypes.c_size_t(ws.numel()), stream)
 
-    def step(pair=None):
+    def step():
+        rc = L.mg_fused_linear_ex(*fused_args)
+        if rc:
+            abi.check(rc, "mg_fused_linear_ex")
+
+    def quant_then_gemm(pair):
+        """The same two kernels through the two separate entry points, with an event pair around the GEMM."""
         abi.reorder_quantize_x(xd, idd, kn, ks, ko, out=aq)
-        if pair:
-            pair[0].record()
+        pair[0].record()
         abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], out=d, w_tiled=True)
-        if pair:
-            pair[1].record()
+        pair[1].record()
 
+    # Clock warm-up by time, whatever --warmup says: the first ~10 ms after an idle period run at other clocks
+    # than the steady state, and the counted warm-up may be a handful of steps.
+    t_warm = time.perf_counter()
+    warm_steps = 0
+    while time.perf_counter() - t_warm < 0.4:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+        warm_steps += 20
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+
+    # Timed region: exactly --steps steps between two synchronizes.  Up to five event marks split it into
+    # sub-loops whose median is reported next to the whole region's mean.
+    nsub = min(5, args.steps)
+    bounds = [round(i * args.steps / nsub) for i in range(nsub + 1)]
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(nsub + 1)]
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(ev[i])
+    for j in range(nsub):
+        marks[j].record()
+        for _ in range(bounds[j], bounds[j + 1]):
+            step()
+    marks[nsub].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    sub_ms = sorted(marks[j].elapsed_time(marks[j + 1]) / (bounds[j + 1] - bounds[j]) for j in range(nsub))
     flops = 2.0 * m * n * k
     value = flops / (ms_per_step * 1e-3) / 1e12
-    gemm_ms = event_ms(ev)
+
+    # The GEMM kernel inside the step: the same two kernels launched through their own entry points with an
+    # event pair around the GEMM (the events cost a few microseconds of device time per step, which is why they
+    # are kept out of the timed region above); five sub-loops, the median of their means.
+    per_sub = max(4, (max(args.steps, 20) + 4) // 5)
+    sub_gemm = []
+    for _ in range(5):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(per_sub)]
+        for pair in ev:
+            quant_then_gemm(pair)
+        torch.cuda.synchronize()
+        sub_gemm.append(event_ms(ev))
+    gemm_ms = sorted(sub_gemm)[2]
     peak = blended_peak(kn, ks, ko)
     gemm_tflops = flops / (gemm_ms * 1e-3) / 1e12
+    t_bytes, t_note = traffic("gemm_c3")
     roofline = {
         "kernel": "mixed GEMM (c3)", "bound": "mfma", "achieved": round(gemm_tflops, 2), "peak": round(peak, 1),
-        "unit": "TFLOP/s", "frac": round(gemm_tflops / peak, 4), "traffic": MEASURED_TRAFFIC.get("gemm_c3"),
+        "unit": "TFLOP/s", "frac": round(gemm_tflops / peak, 4), "traffic": t_bytes, "traffic_source": t_note,
         "avg_kernel_ms": round(gemm_ms, 4), "algorithmic_flops": flops,
+        "protocol": f"clock warm-up {warm_steps} steps (>= 0.4 s), then 5 sub-loops of {per_sub} steps with an event pair "
+                    "around each GEMM launch on the launch stream; median of the sub-loop means",
+        "sub_loop_ms": [round(v, 4) for v in sub_gemm],
     }
 
     extra = {}
     if not args.no_extra:
+        BL = bench_lib()
         # ------------------------------------------------------------ c3 GEMM with the weights as reorder_quantize_w leaves them
         rm, tl = [], []
         for _ in range(5):   # alternate: the chip's clock drifts with load, medians of interleaved runs compare fairly
@@ -219,9 +309,33 @@ def main():
             "workload": "c1 reorder-quantize M=4096 K=4096 (2560/1408/128), random-permutation index, 8 rotating buffer sets, 80 launches replayed as a HIP graph",
             "value": round(q_gbs, 1), "unit": "GB/s", "avg_kernel_ms": round(q_ms, 5),
             "roofline": {"bound": "hbm", "achieved": round(q_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("quant_c1"),
+                         "frac": round(q_gbs / HBM_PEAK_GBS, 4), "traffic": traffic("quant_c1")[0], "traffic_source": traffic("quant_c1")[1],
                          "algorithmic_bytes": qb},
         }
+        # ------------------------------------------------------------ what a plain streaming kernel reaches on c1's bytes
+        # reads the same 33.6 MB per launch from the same rotating inputs and writes 10.6 MB into the same
+        # rotating outputs (one launch of 2048 workgroups of 256, 16 bytes per lane and access), and an empty
+        # launch of the quantizer's grid: the two figures the c1 fraction is to be read against
+        rb, wb = m1 * k1 * 2, (qb - m1 * k1 * 2 - 2 * k1) // 16 * 16
+        st = ctypes.c_void_p(0)
+
+        def stream_copy(i):
+            st.value = torch.cuda.current_stream(dev).cuda_stream
+            rc = BL.mgb_stream(vp(xs[i % nsets]), rb, vp(outs[i % nsets][0]), min(wb, outs[i % nsets][0].numel() // 16 * 16), 2048, st)
+            assert rc == 0
+
+        def empty(i):
+            st.value = torch.cuda.current_stream(dev).cuda_stream
+            assert BL.mgb_empty_launch(1024, 128, st) == 0
+
+        s_ms = graph_ms(stream_copy, iters)
+        e_ms = graph_ms(empty, iters)
+        wrote = min(wb, outs[0][0].numel() // 16 * 16)
+        extra["reorder_quant_c1"]["streaming_reference"] = {
+            "note": "plain streaming kernel on c1's input bytes (same rotation, same graph replay): reads X once, writes "
+                    f"{wrote} bytes; and an empty launch of 1024 workgroups x 128 lanes (the quantizer's launch shape)",
+            "stream_ms": round(s_ms, 5), "stream_gbs": round((rb + wrote) / (s_ms * 1e-3) / 1e9, 1),
+            "empty_launch_ms": round(e_ms, 5)}
         # ------------------------------------------------------------ c1 with an RMSNorm fused into the row pass
         gamma1 = torch.ones(k1, dtype=torch.bfloat16, device=dev)
         n_ms = graph_ms(lambda i: abi.rmsnorm_reorder_quantize_x(xs[i % nsets], gamma1, 1e-5, idx1, kn1, ks1, ko1,
@@ -241,7 +355,7 @@ def main():
             "workload": "reorder index of the c1 activations: per-channel absmax over M=4096 rows + sort of K=4096 channels",
             "value": round(cb / (c_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "avg_ms": round(c_ms, 5),
             "roofline": {"bound": "hbm", "achieved": round(cb / (c_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(cb / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("calibrate_c1"),
+                         "frac": round(cb / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": traffic("calibrate_c1")[0], "traffic_source": traffic("calibrate_c1")[1],
                          "algorithmic_bytes": cb},
         }
         del xs, outs, base
@@ -270,7 +384,7 @@ def main():
             "value": round(g_gbs, 1), "unit": "GB/s", "avg_kernel_ms": round(g_ms, 5),
             "tflops": round(2.0 * m2 * n2 * k2 / (g_ms * 1e-3) / 1e12, 3),
             "roofline": {"bound": "hbm", "achieved": round(g_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(g_gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("decode_c2"),
+                         "frac": round(g_gbs / HBM_PEAK_GBS, 4), "traffic": traffic("decode_c2")[0], "traffic_source": traffic("decode_c2")[1],
                          "algorithmic_bytes": gb},
         }
         del wq
@@ -279,7 +393,8 @@ def main():
         # fused step (activation reorder-quantize + mixed GEMM) per shape; weights quantized outside the timing
         from mixedgemm_amd import linear as caller
         matrix = []
-        shapes = [("c0", 128, 4096, 4096), ("c4", 2048, 4096, 14336), ("", 4096, 13824, 5120), ("", 4096, 5120, 13824),
+        shapes = [("c0", 128, 4096, 4096), ("c4", 2048, 4096, 14336), ("reference bench_gemm.cu:23-27", 1024, 4096, 4096),
+                  ("", 4096, 13824, 5120), ("", 4096, 5120, 13824),
                   ("", 4096, 18944, 3584), ("", 4096, 3584, 18944), ("", 4096, 4096, 12288)]
         for tag, mm, nn, kk in shapes:
             knm, ksm, kom = caller.default_split(kk)
@@ -305,6 +420,7 @@ def main():
                            "quant_ms": round(times[0], 5), "gemm_ms": round(times[1], 5),
                            "gemm_tflops": round(flops / (times[1] * 1e-3) / 1e12, 1),
                            "fused_tflops": round(flops / ((times[0] + times[1]) * 1e-3) / 1e12, 1),
+                           "gemm_frac_of_peak": round(flops / (times[1] * 1e-3) / 1e12 / blended_peak(knm, ksm, kom), 4),
                            "quant_gbs": round(quant_bytes(mm, kk, knm, ksm, kom) / (times[0] * 1e-3) / 1e9, 1)})
             del xm, wqm, aqm, dm
         extra["shape_matrix"] = {"note": "back-to-back launches on one buffer set (operands may sit in the 256 MB "
@@ -346,8 +462,8 @@ def main():
         # ------------------------------------------------------------ what the matrix cores sustain on this box
         # register-resident scaled-MFMA loop on all CUs: with pseudo-random operand bits the chip hits its
         # power limit and clocks down, which bounds any GEMM on real data below the nominal peak
-        c_tf, c_ghz = abi.measure_mfma_ceiling(False)
-        r_tf, r_ghz = abi.measure_mfma_ceiling(True)
+        c_tf, c_ghz = measure_mfma_ceiling(BL, False)
+        r_tf, r_ghz = measure_mfma_ceiling(BL, True)
         extra["mfma_e2m1_register_loop"] = {
             "constant_operands": {"tflops": round(c_tf, 1), "shader_ghz": round(c_ghz, 3)},
             "random_operands": {"tflops": round(r_tf, 1), "shader_ghz": round(r_ghz, 3)},
@@ -409,10 +525,12 @@ def main():
     out = {
         "metric": "mixed_mx_gemm_tflops", "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_sub_loops": [round(v, 4) for v in sub_ms], "ms_per_step_median_sub_loop": round(sub_ms[len(sub_ms) // 2], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "mxfp4/mxfp6/mxfp8 x mxfp4 -> f32 accumulate -> bf16", "data": "synthetic",
         "config": {"workload": "c3 prefill: reorder-quantize bf16 X[4096,4096] + mixed GEMM vs MXFP4 W[14336,4096] "
-                               "(K split 2560 fp4 / 1408 fp6 / 128 fp8), bf16 out; weight codes packed tile-major offline",
+                               "(K split 2560 fp4 / 1408 fp6 / 128 fp8), bf16 out; weight codes packed tile-major offline; "
+                               "one mg_fused_linear_ex call per step",
                    "M": m, "N": n, "K": k, "KN": kn, "KS": ks, "KO": ko},
         "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
     }

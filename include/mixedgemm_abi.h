@@ -3,7 +3,8 @@
  *
  * Plain C types only: device pointers, sizes, a HIP stream passed as void*.
  * Every entry point validates its arguments on the host, enqueues its kernels
- * on `stream` and returns without synchronizing; none allocates.  The return
+ * on `stream` and returns without synchronizing (mg_device_synchronize and
+ * mg_check_reorder_index, whose job it is to wait, excepted); none allocates.  The return
  * value is a status code: 0 on success, a hipError_t value for a HIP failure, or
  * one of the MG_ERR_* codes below.  mg_status_string() names any of them.
  *
@@ -23,7 +24,7 @@ extern "C" {
 #define MG_OK 0
 #define MG_ERR_BAD_SHAPE 10001   /* a segment is not a multiple of 32, K mismatch, negative size */
 #define MG_ERR_BAD_POINTER 10002 /* null or insufficiently aligned pointer (16 bytes required) */
-#define MG_ERR_BAD_INDEX 10003   /* reorder index entry outside [0, K) (only when checked on host) */
+#define MG_ERR_BAD_INDEX 10003   /* reorder index entry outside [0, K): mg_check_reorder_index[_host] */
 #define MG_ERR_UNSUPPORTED 10004 /* shape outside what the kernels handle (K > 32736) */
 
 /* Operand selector for mg_sf_bytes(). */
@@ -162,19 +163,22 @@ int mg_calibrate_reorder_index(const void* x_bf16, int M, int K, int16_t* idx,
                                void* workspace, size_t workspace_bytes, void* stream);
 size_t mg_calibrate_workspace_bytes(int K);
 
+/* Range check of a reorder index, for the places where an index enters the system (calibration, a
+ * pack file, a caller's own tensor): MG_OK when every entry lies in [0, K), MG_ERR_BAD_INDEX otherwise.
+ * The reference never checks: its K is a template constant and an out-of-range entry reads outside the
+ * staged row (src/reorder.cu:154-158, 187).  The quantizers here clamp such an entry to channel K - 1, so
+ * that they stay inside the row whatever the index holds; these calls are how a caller finds out.
+ *   _host: idx is host memory.  The other: idx is device memory; copies it to the host behind the work
+ *   already enqueued on `stream` and BLOCKS until that copy has finished (a pack-time call). */
+int mg_check_reorder_index_host(const int16_t* idx, int K);
+int mg_check_reorder_index(const int16_t* idx, int K, void* stream);
+
 /* Blocks the host until all work on the current device has finished
  * (src/bindings.cpp:59,178,297 do this after every operator). */
 int mg_device_synchronize(void);
 
 /* Text for a status code returned by any function above. */
 const char* mg_status_string(int status);
-
-/* Measurement helper with no counterpart in the reference (bench.py reports it next to the
- * roofline): rate and shader clock at which the whole GPU sustains the E2M1 x E2M1 scaled MFMA
- * from registers, over `iters` x 16 instructions per wave, with constant (0) or pseudo-random
- * (1) operand bits.  Allocates and frees its own small buffers, runs on the default stream and
- * blocks until done.  Returns 0 or a hipError_t. */
-int mg_measure_mfma_ceiling(int random_operands, int iters, double* tflops, double* shader_ghz);
 
 #ifdef __cplusplus
 }

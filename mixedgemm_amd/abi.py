@@ -23,7 +23,7 @@ SYMBOLS = (
     "mg_weights_tileable", "mg_fused_linear_ex", "mg_rmsnorm_reorder_quantize_x", "mg_fused_norm_linear",
     "mg_fused_linear",
     "mg_fused_workspace_bytes", "mg_sf_bytes", "mg_sf_offset", "mg_device_synchronize", "mg_status_string",
-    "mg_measure_mfma_ceiling", "mg_calibrate_reorder_index", "mg_calibrate_workspace_bytes",
+    "mg_calibrate_reorder_index", "mg_calibrate_workspace_bytes", "mg_check_reorder_index", "mg_check_reorder_index_host",
 )
 
 _lib = None
@@ -66,8 +66,8 @@ def lib() -> ctypes.CDLL:
         L.mg_device_synchronize.restype, L.mg_device_synchronize.argtypes = i, []
         L.mg_calibrate_reorder_index.restype, L.mg_calibrate_reorder_index.argtypes = i, [p, i, i, p, p, z, p]
         L.mg_calibrate_workspace_bytes.restype, L.mg_calibrate_workspace_bytes.argtypes = z, [i]
-        L.mg_measure_mfma_ceiling.restype = i
-        L.mg_measure_mfma_ceiling.argtypes = [i, i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+        L.mg_check_reorder_index.restype, L.mg_check_reorder_index.argtypes = i, [p, i, p]
+        L.mg_check_reorder_index_host.restype, L.mg_check_reorder_index_host.argtypes = i, [p, i]
         L.mg_status_string.restype, L.mg_status_string.argtypes = ctypes.c_char_p, [i]
         _lib = L
     return _lib
@@ -226,6 +226,14 @@ def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None
         raise MixedGemmError("the three segments of an operand must have the same number of rows")
     if bn.shape[1] * 2 != kn or bs.shape[1] * 2 != ks or bo.shape[1] * 2 != ko:
         raise MixedGemmError("activation and weight segments disagree on KN / KS / KO")
+    for t in (bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out):
+        if t.device != an.device:
+            raise MixedGemmError("all operands must be on the same GPU")
+    for name, t, rows, kseg, operand in (("SFAN", sfan, m, kn, MG_OPERAND_A), ("SFAS", sfas, m, ks, MG_OPERAND_A),
+                                         ("SFAO", sfao, m, ko, MG_OPERAND_A), ("SFBN", sfbn, n, kn, MG_OPERAND_B),
+                                         ("SFBS", sfbs, n, ks, MG_OPERAND_B), ("SFBO", sfbo, n, ko, MG_OPERAND_B)):
+        if t.numel() < sf_bytes(rows, kseg, operand):
+            raise MixedGemmError(f"{name}: {t.numel()} bytes, need {sf_bytes(rows, kseg, operand)}")
     # rows the activation buffers are readable for: whole tiles if every storage has the room
     r = padded_rows(m)
     roomy = all(_capacity(t) >= r * t.shape[1] for t in (an, as_, ao)) and all(
@@ -238,13 +246,46 @@ def matmul(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, out=None
     return out
 
 
+def _check_weights(x, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko):
+    """The six weight tensors of a fused call: uint8, contiguous, on x's GPU, [N, kseg / 2] codes and scale
+    buffers of at least the size the GEMM reads.  Returns N."""
+    for name, t in (("BN", bn), ("BS", bs), ("BO", bo), ("SFBN", sfbn), ("SFBS", sfbs), ("SFBO", sfbo)):
+        _require(t, torch.uint8, name)
+        if t.device != x.device:
+            raise MixedGemmError(f"{name}: on {t.device}, X is on {x.device}")
+    for name, t in (("BN", bn), ("BS", bs), ("BO", bo)):
+        if t.dim() != 2:
+            raise MixedGemmError(f"{name}: expected a 2-D tensor")
+    n = bn.shape[0]
+    for name, t, kseg in (("BN", bn, kn), ("BS", bs, ks), ("BO", bo, ko)):
+        if tuple(t.shape) != (n, kseg // 2):
+            raise MixedGemmError(f"{name}: expected shape {(n, kseg // 2)}, got {tuple(t.shape)}")
+    for name, t, kseg in (("SFBN", sfbn, kn), ("SFBS", sfbs, ks), ("SFBO", sfbo, ko)):
+        if t.numel() < sf_bytes(n, kseg, MG_OPERAND_B):
+            raise MixedGemmError(f"{name}: {t.numel()} bytes, need {sf_bytes(n, kseg, MG_OPERAND_B)}")
+    return n
+
+
+def _check_fused_inputs(x, reorder_index, kn, ks, ko):
+    _require(x, torch.bfloat16, "X")
+    _require(reorder_index, torch.int16, "reorder_index")
+    if x.dim() != 2:
+        raise MixedGemmError("X: expected a 2-D tensor")
+    if min(kn, ks, ko) < 0 or (kn | ks | ko) % 32:
+        raise MixedGemmError("KN, KS, KO must be non-negative multiples of 32")
+    if x.shape[1] != kn + ks + ko or reorder_index.numel() != x.shape[1]:
+        raise MixedGemmError(f"X has {x.shape[1]} channels, the split sums to {kn + ks + ko}, the index has {reorder_index.numel()}")
+    if reorder_index.device != x.device:
+        raise MixedGemmError(f"reorder_index: on {reorder_index.device}, X is on {x.device}")
+
+
 def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, workspace=None, out=None, w_tiled=False,
                  norm_weight=None, eps=0.0):
     """Activation reorder-quantize + mixed GEMM on one stream; returns bf16 [M, N].  With norm_weight
     (bf16 [K]) the activations pass through an RMSNorm first, inside the quantizer's row pass."""
-    _require(x, torch.bfloat16, "X")
-    _require(reorder_index, torch.int16, "reorder_index")
-    m, n = x.shape[0], bn.shape[0]
+    _check_fused_inputs(x, reorder_index, kn, ks, ko)
+    m = x.shape[0]
+    n = _check_weights(x, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko)
     need = fused_workspace_bytes(m, kn, ks, ko)
     if workspace is None:
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
@@ -252,20 +293,33 @@ def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, wor
         out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     else:
         _check_out(out, (m, n), torch.bfloat16, "out")
-    if x.shape[1] != kn + ks + ko or reorder_index.numel() != x.shape[1]:
-        raise MixedGemmError(f"X has {x.shape[1]} channels, the split sums to {kn + ks + ko}, the index has {reorder_index.numel()}")
-    if workspace.numel() < need or not workspace.is_cuda or workspace.dtype != torch.uint8:
-        raise MixedGemmError(f"workspace: need {need} uint8 on the GPU")
+    _require(workspace, torch.uint8, "workspace")
+    if workspace.numel() < need or workspace.device != x.device or out.device != x.device:
+        raise MixedGemmError(f"workspace: need {need} uint8 on X's GPU (and `out` there too)")
     if norm_weight is not None:
         _require(norm_weight, torch.bfloat16, "norm_weight")
-        if norm_weight.numel() != x.shape[1]:
-            raise MixedGemmError(f"norm_weight must have {x.shape[1]} entries")
+        if norm_weight.numel() != x.shape[1] or norm_weight.device != x.device:
+            raise MixedGemmError(f"norm_weight must have {x.shape[1]} entries on X's GPU")
     status = lib().mg_fused_norm_linear(_ptr(x), _ptr(norm_weight), float(eps), _ptr(reorder_index), _ptr(bn), _ptr(bs),
                                         _ptr(bo), _ptr(sfbn), _ptr(sfbs), _ptr(sfbo), m, n, kn, ks, ko,
                                         MG_FLAG_W_TILED if w_tiled else 0,
                                         _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
     check(status, "mg_fused_norm_linear")
     return out
+
+
+def check_reorder_index(reorder_index, k=None) -> None:
+    """Raises MixedGemmError unless every entry of the int16 index lies in [0, K).  Blocks for a GPU tensor."""
+    if reorder_index.dtype != torch.int16 or not reorder_index.is_contiguous():
+        raise MixedGemmError("reorder_index: expected a contiguous int16 tensor")
+    k = reorder_index.numel() if k is None else int(k)
+    if reorder_index.numel() != k:
+        raise MixedGemmError(f"reorder_index has {reorder_index.numel()} entries, expected {k}")
+    if reorder_index.is_cuda:
+        status = lib().mg_check_reorder_index(_ptr(reorder_index), k, _stream(reorder_index))
+    else:
+        status = lib().mg_check_reorder_index_host(ctypes.c_void_p(reorder_index.data_ptr()), k)
+    check(status, "mg_check_reorder_index")
 
 
 def weights_tileable(n: int, kn: int, ks: int, ko: int) -> bool:
@@ -302,14 +356,6 @@ def calibrate_reorder_index(x, out=None, workspace=None):
     check(lib().mg_calibrate_reorder_index(_ptr(x), m, k, _ptr(out), _ptr(workspace), workspace.numel(),
                                            _stream(x)), "mg_calibrate_reorder_index")
     return out
-
-
-def measure_mfma_ceiling(random_operands: bool, iters: int = 4000):
-    """(TFLOP/s, shader GHz) of a register-resident E2M1 x E2M1 scaled-MFMA loop on all CUs."""
-    tf, ghz = ctypes.c_double(0.0), ctypes.c_double(0.0)
-    check(lib().mg_measure_mfma_ceiling(int(bool(random_operands)), iters, ctypes.byref(tf), ctypes.byref(ghz)),
-          "mg_measure_mfma_ceiling")
-    return tf.value, ghz.value
 
 
 def device_synchronize() -> None:

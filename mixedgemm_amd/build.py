@@ -5,6 +5,7 @@
 
 Outputs (kept out of git, shipped with the tree):
     mixedgemm_amd/lib/libmixedgemm_hip.so   hand-written gfx950 kernels + extern "C" entry points
+    mixedgemm_amd/lib/libmixedgemm_bench.so measurement kernels bench.py times next to the library (not the product)
     build/mixedgemm.so                      torch extension with the reference's operator surface
     build/abi_driver                        torch-free host program (tests/c_host) on the C-ABI
 """
@@ -25,11 +26,15 @@ EXT_PATH = os.path.join(EXT_DIR, "mixedgemm.so")
 DRIVER_SRC = os.path.join(ROOT, "tests", "c_host", "abi_driver.cpp")
 DRIVER_PATH = os.path.join(EXT_DIR, "abi_driver")
 
-HIP_SOURCES = ["abi.hip", "reorder_quant.hip", "mixed_gemm.hip", "mixed_gemm_256.hip", "calibrate.hip", "ceiling.hip"]
+BENCH_LIB_PATH = os.path.join(LIB_DIR, "libmixedgemm_bench.so")
+OBJ_DIR = os.path.join(EXT_DIR, "obj")
+
+HIP_SOURCES = ["abi.hip", "reorder_quant.hip", "mixed_gemm.hip", "mixed_gemm_256.hip", "calibrate.hip"]
+BENCH_SOURCES = ["bench_kernels.hip"]
 HIP_HEADERS = ["mg_common.h", os.path.join(ROOT, "include", "mixedgemm_abi.h")]
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed FP32 VALU forms are kept out of every kernel
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
@@ -43,16 +48,42 @@ def _stale(target: str, deps: list[str]) -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build_hip_library(force: bool = False, verbose: bool = False) -> str:
-    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    deps = srcs + [h if os.path.isabs(h) else os.path.join(CSRC, h) for h in HIP_HEADERS]
-    if force or _stale(LIB_PATH, deps):
-        os.makedirs(LIB_DIR, exist_ok=True)
-        cmd = ["hipcc", *HIPCC_FLAGS, "-o", LIB_PATH, *srcs]
+def _compile_and_link(sources: list[str], target: str, force: bool, verbose: bool) -> str:
+    """One object per source, compiled side by side, then one link."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    srcs = [os.path.join(CSRC, s) for s in sources]
+    hdrs = [h if os.path.isabs(h) else os.path.join(CSRC, h) for h in HIP_HEADERS]
+    os.makedirs(LIB_DIR, exist_ok=True)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = [os.path.join(OBJ_DIR, os.path.basename(s) + ".o") for s in srcs]
+
+    def compile_one(pair):
+        src, obj = pair
+        if force or _stale(obj, [src] + hdrs):
+            cmd = ["hipcc", *HIPCC_FLAGS, "-c", src, "-o", obj]
+            if verbose:
+                print(" ".join(cmd), flush=True)
+            subprocess.check_call(cmd)
+
+    with ThreadPoolExecutor(max_workers=min(len(srcs), 6)) as pool:
+        list(pool.map(compile_one, zip(srcs, objs)))
+    if force or _stale(target, objs):
+        cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", target, *objs]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
-    return LIB_PATH
+    return target
+
+
+def build_hip_library(force: bool = False, verbose: bool = False) -> str:
+    return _compile_and_link(HIP_SOURCES, LIB_PATH, force, verbose)
+
+
+def build_bench_library(force: bool = False, verbose: bool = False) -> str:
+    """Measurement kernels for bench.py (MFMA register loop, plain copy, empty launch): their own
+    shared object, so that the product library holds the hot path only."""
+    return _compile_and_link(BENCH_SOURCES, BENCH_LIB_PATH, force, verbose)
 
 
 def build_torch_extension(force: bool = False, verbose: bool = False) -> str:
@@ -98,6 +129,7 @@ def build_c_host_driver(force: bool = False, verbose: bool = False) -> str:
 
 def build_all(force: bool = False, verbose: bool = False) -> None:
     build_hip_library(force, verbose)
+    build_bench_library(force, verbose)
     build_torch_extension(force, verbose)
     build_c_host_driver(force, verbose)
 

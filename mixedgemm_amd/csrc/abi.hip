@@ -1,9 +1,11 @@
 // extern "C" surface of the library: argument validation on the host, then the
-// kernel launchers.  Nothing here allocates or synchronizes (except
-// mg_device_synchronize, whose only job that is).
+// kernel launchers.  Nothing here allocates device memory or synchronizes (except
+// mg_device_synchronize and mg_check_reorder_index, whose job that is).
 #include "../../include/mixedgemm_abi.h"
 
 #include "mg_common.h"
+
+#include <vector>
 
 namespace mg {
 template <bool IS_W>
@@ -176,6 +178,27 @@ int mg_calibrate_reorder_index(const void* x_bf16, int M, int K, int16_t* idx, v
   if (!x_bf16 || !aligned16(x_bf16) || !idx || !workspace || !aligned16(workspace)) return MG_ERR_BAD_POINTER;
   if (workspace_bytes < mg::calibrate_workspace_bytes(K)) return MG_ERR_BAD_SHAPE;
   return (int)mg::launch_calibrate(x_bf16, M, K, idx, workspace, static_cast<hipStream_t>(stream));
+}
+
+int mg_check_reorder_index_host(const int16_t* idx, int K) {
+  if (K < 0) return MG_ERR_BAD_SHAPE;
+  if (K > 0 && idx == nullptr) return MG_ERR_BAD_POINTER;
+  for (int i = 0; i < K; ++i)
+    if (idx[i] < 0 || idx[i] >= K) return MG_ERR_BAD_INDEX;
+  return MG_OK;
+}
+
+int mg_check_reorder_index(const int16_t* idx, int K, void* stream) {
+  if (K < 0) return MG_ERR_BAD_SHAPE;
+  if (K > 32767) return MG_ERR_UNSUPPORTED;
+  if (K == 0) return MG_OK;
+  if (idx == nullptr) return MG_ERR_BAD_POINTER;
+  std::vector<int16_t> host((size_t)K);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipError_t e = hipMemcpyAsync(host.data(), idx, (size_t)K * sizeof(int16_t), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return (int)e;
+  return mg_check_reorder_index_host(host.data(), K);
 }
 
 int mg_device_synchronize(void) { return (int)hipDeviceSynchronize(); }

@@ -1,4 +1,8 @@
-// Measurement helper, not part of the hot path: the rate at which all 1024 SIMDs of the GPU
+// Measurement kernels for bench.py, built into their own shared object (libmixedgemm_bench.so): none
+// of this is part of the hot path or of the product library, and unlike the product's entry points
+// mgb_measure_mfma_ceiling allocates, uses the default stream and blocks.
+//
+// mgb_measure_mfma_ceiling: the rate at which all 1024 SIMDs of the GPU
 // sustain v_mfma_scale_f32_32x32x64_f8f6f4 (E2M1 x E2M1) from registers, with nothing else in the
 // loop.  Operand bits are either small constants or pseudo-random: with random bits the
 // chip runs into its power limit and clocks down, so the second figure is the ceiling a GEMM on
@@ -56,12 +60,50 @@ __global__ void __launch_bounds__(256) mfma_ceiling_kernel(float* __restrict__ o
   if (threadIdx.x == 0) cycles[blockIdx.x] = t1 - t0;
 }
 
+// Streaming reference for the memory-bound kernels: reads `nread` 16-byte pieces once, writes `nwrite`
+// pieces once, nothing else (the reads are folded into the value written so that they are not dropped).
+__global__ void __launch_bounds__(256) stream_kernel(const v4u* __restrict__ src, size_t nread, v4u* __restrict__ dst,
+                                                     size_t nwrite) {
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x, step = (size_t)gridDim.x * 256;
+  v4u acc = {0u, 0u, 0u, 0u};
+  for (size_t i = t; i < nread; i += 4 * step) {
+    v4u v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = src[min(i + u * step, nread - 1)];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc ^= v[u];
+  }
+  for (size_t i = t; i < nwrite; i += step) __builtin_nontemporal_store(acc, dst + i);
+}
+
+__global__ void __launch_bounds__(1024) empty_kernel(int* __restrict__ sink) {
+  if (sink != nullptr && threadIdx.x == 1023 && blockIdx.x == 0x7fffffff) *sink = 0;
+}
+
 }  // namespace
 
 }  // namespace mg
 
+// Reads read_bytes from src and writes write_bytes to dst (multiples of 16) with `workgroups` workgroups of 256.
 extern "C" __attribute__((visibility("default")))
-int mg_measure_mfma_ceiling(int random_operands, int iters, double* tflops, double* shader_ghz) {
+int mgb_stream(const void* src, size_t read_bytes, void* dst, size_t write_bytes, int workgroups, void* stream) {
+  if (workgroups <= 0 || (read_bytes & 15) || (write_bytes & 15)) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(mg::stream_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const mg::v4u*>(src), read_bytes / 16, static_cast<mg::v4u*>(dst), write_bytes / 16);
+  return (int)hipGetLastError();
+}
+
+// A launch of `workgroups` x `threads` that does nothing: what a launch of that size costs by itself.
+extern "C" __attribute__((visibility("default")))
+int mgb_empty_launch(int workgroups, int threads, void* stream) {
+  if (workgroups <= 0 || threads <= 0 || threads > 1024) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(mg::empty_kernel, dim3(workgroups), dim3(threads), 0, static_cast<hipStream_t>(stream),
+                     static_cast<int*>(nullptr));
+  return (int)hipGetLastError();
+}
+
+extern "C" __attribute__((visibility("default")))
+int mgb_measure_mfma_ceiling(int random_operands, int iters, double* tflops, double* shader_ghz) {
   constexpr int kGrid = 256;   // one workgroup of 4 waves per CU
   float* out = nullptr;
   long long* cyc = nullptr;
@@ -74,10 +116,10 @@ int mg_measure_mfma_ceiling(int random_operands, int iters, double* tflops, doub
   long long host_cyc[kGrid];
   if (e == hipSuccess) {
     for (int rep = 0; rep < 2 && e == hipSuccess; ++rep) {   // first launch warms up clocks and code
-      hipEventRecord(a, nullptr);
+      (void)hipEventRecord(a, nullptr);
       if (random_operands) hipLaunchKernelGGL(mg::mfma_ceiling_kernel<true>, dim3(kGrid), dim3(256), 0, nullptr, out, iters, cyc);
       else hipLaunchKernelGGL(mg::mfma_ceiling_kernel<false>, dim3(kGrid), dim3(256), 0, nullptr, out, iters, cyc);
-      hipEventRecord(b, nullptr);
+      (void)hipEventRecord(b, nullptr);
       e = hipEventSynchronize(b);
     }
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, a, b);
@@ -91,9 +133,9 @@ int mg_measure_mfma_ceiling(int random_operands, int iters, double* tflops, doub
     *tflops = flops / (ms * 1e-3) / 1e12;
     *shader_ghz = avg / (ms * 1e6);
   }
-  if (a) hipEventDestroy(a);
-  if (b) hipEventDestroy(b);
-  if (out) hipFree(out);
-  if (cyc) hipFree(cyc);
+  if (a) (void)hipEventDestroy(a);
+  if (b) (void)hipEventDestroy(b);
+  if (out) (void)hipFree(out);
+  if (cyc) (void)hipFree(cyc);
   return (int)e;
 }

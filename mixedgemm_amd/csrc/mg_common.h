@@ -60,4 +60,25 @@ inline hipError_t allow_dynamic_lds(const void* kernel, int bytes) {
   return e;
 }
 
+// LDS bytes a workgroup may use and the number of CUs of the current device (asked once per device).
+struct DeviceLimits { int lds_bytes, cus; };
+inline hipError_t device_limits(DeviceLimits* out) {
+  static std::mutex mu;
+  static DeviceLimits table[64] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (table[dev].cus == 0) {
+    int lds = 0, cus = 0;
+    e = hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    table[dev] = DeviceLimits{lds, cus};
+  }
+  *out = table[dev];
+  return hipSuccess;
+}
+
 }  // namespace mg

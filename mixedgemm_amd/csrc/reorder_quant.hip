@@ -177,13 +177,14 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
     for (int it = 0; it < 4; ++it)
       gv[it] = *reinterpret_cast<const v4u*>(gamma + (size_t)min(tid + it * nthr, nchunks - 1) * 8);
   }
-  // Byte offsets of the lane's 32 gathered channels inside a tile (the same for every row).
+  // Byte offsets of the lane's 32 gathered channels inside a tile (the same for every row).  An entry outside
+  // [0, K) is read as channel K - 1, so that the gather stays inside the tile whatever the index holds.
   unsigned ga[32];
 #pragma unroll
   for (int q = 0; q < 4; ++q)
 #pragma unroll
     for (int e = 0; e < 8; ++e)
-      ga[q * 8 + e] = ((e & 1) ? (iv[q][e >> 1] >> 16) : (iv[q][e >> 1] & 0xffffu)) * (2 * R);
+      ga[q * 8 + e] = min((e & 1) ? (iv[q][e >> 1] >> 16) : (iv[q][e >> 1] & 0xffffu), (unsigned)(K - 1)) * (2 * R);
 
   // The loop body exists once per LDS buffer, so that the buffer's offset is a compile-time
   // constant wherever the buffers are a fixed distance apart (kFixed) and folds into the LDS
@@ -327,34 +328,36 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
   const uint16_t* gm = static_cast<const uint16_t*>(gamma);
   const int threads = ((K >> 5) + 63) & ~63;
   const uint16_t* xb = static_cast<const uint16_t*>(x);
+  DeviceLimits lim;
+  if (hipError_t e = device_limits(&lim); e != hipSuccess) return e;
+  hipError_t err = hipSuccess;
   // R rows interleaved in LDS.  More row groups than `resident` workgroups: each workgroup
   // streams several groups through a double-buffered tile.
   auto launch = [&](auto kernel, int R) {
     const int tile = K * 2 * R;
     const int ngroups = ceil_div(rows, R);
-#ifndef MG_QUANT_WGS_PER_CU
-#define MG_QUANT_WGS_PER_CU 4
-#endif
     // second LDS buffer: a fixed 16 KB * R behind the first for the 256-lane kernels (see kFixed), else one tile behind
     const int second = K <= 8192 ? 256 * 64 * R : tile;
-    int per_cu = (160 * 1024) / (second + tile);
-    per_cu = per_cu < 1 ? 1 : (per_cu > MG_QUANT_WGS_PER_CU ? MG_QUANT_WGS_PER_CU : per_cu);
-    const int resident = 256 * per_cu;
-    const bool stream_groups = ngroups > resident && second + tile <= 160 * 1024;
+    int per_cu = lim.lds_bytes / (second + tile);
+    per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+    const int resident = lim.cus * per_cu;
+    const bool stream_groups = ngroups > resident && second + tile <= lim.lds_bytes;
     const int grid = stream_groups ? resident : ngroups;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), (size_t)(stream_groups ? second + tile : tile), stream, xb, idx, rows, K,
+    const int lds = stream_groups ? second + tile : tile;
+    if (lds > lim.lds_bytes) { err = hipErrorInvalidValue; return; }
+    err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), lim.lds_bytes);
+    if (err != hipSuccess) return;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), (size_t)lds, stream, xb, idx, rows, K,
                        KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream_groups ? tile : 0, gm, eps);
+    err = hipGetLastError();
   };
-#ifndef MG_QUANT_R_SMALLK
-#define MG_QUANT_R_SMALLK 1
-#endif
-  constexpr int R = MG_QUANT_R_SMALLK;
+  constexpr int R = 1;
   if constexpr (!IS_W) {
     if (gamma != nullptr) {
       if (K <= 8192) launch(reorder_quant_kernel<R, false, 256, true>, R);
       else if (K <= 16384) launch(reorder_quant_kernel<2, false, 512, true>, 2);
       else launch(reorder_quant_kernel<1, false, 1024, true>, 1);
-      return hipGetLastError();
+      return err;
     }
   }
   if (K <= 8192) {
@@ -364,7 +367,7 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
   } else {
     launch(reorder_quant_kernel<1, IS_W, 1024, false>, 1);
   }
-  return hipGetLastError();
+  return err;
 }
 
 template hipError_t launch_reorder_quant<false>(const void*, const int16_t*, int, int, int, int, int, uint8_t*, uint8_t*,

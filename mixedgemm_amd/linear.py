@@ -82,6 +82,7 @@ class PackedWeights:
         bindings.cpp:188-305); with `tile`, shapes that allow it are then put in tile-major order."""
         split = tuple(split) if split is not None else default_split(weight.shape[1])
         n = weight.shape[0]
+        abi.check_reorder_index(reorder_index, weight.shape[1])
         # the whole-tile kernel wants a multiple of 256 features: zero rows are cheap, the layer drops their outputs
         if tile and n > 256 and n % 256 and abi.weights_tileable((n + 255) // 256 * 256, *split):
             pad = torch.zeros(((n + 255) // 256 * 256 - n, weight.shape[1]), dtype=weight.dtype, device=weight.device)
@@ -175,6 +176,13 @@ class PackedWeights:
                 raise ValueError(f"{name}: expected at least {need} uint8, got {t.numel()} {t.dtype}")
         if self.reorder_index.dtype != torch.int16 or self.reorder_index.numel() != kn + ks + ko:
             raise ValueError("reorder_index: expected int16 [K]")
+        devices = {t.device for t in (*self.tensors(), self.reorder_index)}
+        if len(devices) != 1:
+            raise ValueError(f"tensors on different devices: {sorted(str(d) for d in devices)}")
+        try:
+            abi.check_reorder_index(self.reorder_index.contiguous(), kn + ks + ko)   # blocks for GPU tensors: a pack-time check
+        except abi.MixedGemmError as e:
+            raise ValueError(str(e)) from e
         if self.tiled and not self.tileable():
             raise ValueError("tile-major codes for a shape that cannot be tiled")
 

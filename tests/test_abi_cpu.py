@@ -138,3 +138,139 @@ def test_extension_module_surface():
         mixedgemm.reorder_quantize_x(x, idx, 50, 30, 20, 2, 2)
     with pytest.raises(RuntimeError, match="Value error in run_reorder_bf16_fp4"):
         mixedgemm.reorder_quantize_w(x, idx, 50, 30, 20, 2, 2)
+
+
+# ------------------------------------------------------------------ reorder index range, host side
+def test_check_reorder_index_host(abi):
+    import torch
+    k = 256
+    good = torch.randperm(k).to(torch.int16)
+    abi.check_reorder_index(good)
+    assert abi.lib().mg_check_reorder_index_host(ctypes.c_void_p(good.data_ptr()), k) == 0
+    for pos, val in ((0, -1), (17, k), (255, 32767), (3, -32768)):
+        bad = good.clone()
+        bad[pos] = val
+        assert abi.lib().mg_check_reorder_index_host(ctypes.c_void_p(bad.data_ptr()), k) == 10003
+        with pytest.raises(abi.MixedGemmError, match="out of range"):
+            abi.check_reorder_index(bad)
+    with pytest.raises(abi.MixedGemmError):
+        abi.check_reorder_index(good, k + 32)
+    with pytest.raises(abi.MixedGemmError):
+        abi.check_reorder_index(good.to(torch.int32))
+    # repeats are a legal gather
+    abi.check_reorder_index(torch.zeros(k, dtype=torch.int16))
+    assert abi.lib().mg_check_reorder_index_host(ctypes.c_void_p(0), 0) == 0
+    assert abi.lib().mg_check_reorder_index_host(ctypes.c_void_p(0), 32) == 10002
+    assert "out of range" in abi.status_string(10003)
+
+
+# ------------------------------------------------------------------ operand checks of the Python binding
+class _NoLaunch:
+    """Stands in for the loaded library: size queries go through, any compute entry point fails the test."""
+
+    def __init__(self, real):
+        self._real = real
+
+    def __getattr__(self, name):
+        if name in ("mg_sf_bytes", "mg_sf_offset", "mg_fused_workspace_bytes", "mg_padded_rows", "mg_status_string",
+                    "mg_weights_tileable", "mg_calibrate_workspace_bytes", "mg_check_reorder_index_host"):
+            return getattr(self._real, name)
+        raise AssertionError(f"{name} reached with operands that should have been refused")
+
+
+@pytest.fixture
+def no_launch(abi, monkeypatch):
+    """The binding with its GPU requirement lifted (CPU tensors pass the device check) and every launch
+    turned into a test failure: what is left is the validation that runs before a launch."""
+    import torch
+    real = abi.lib()
+    fake = _NoLaunch(real)
+    monkeypatch.setattr(abi, "lib", lambda: fake)
+
+    def require(t, dtype, name):
+        if t.dtype != dtype:
+            raise abi.MixedGemmError(f"{name}: expected {dtype}, got {t.dtype}")
+        if not t.is_contiguous():
+            raise abi.MixedGemmError(f"{name}: expected a contiguous tensor")
+
+    monkeypatch.setattr(abi, "_require", require)
+    monkeypatch.setattr(abi, "_stream", lambda t: ctypes.c_void_p(0))
+    return abi
+
+
+def _weights(abi, n, kn, ks, ko):
+    import torch
+    u8 = dict(dtype=torch.uint8)
+    return [torch.zeros((n, kn // 2), **u8), torch.zeros((n, ks // 2), **u8), torch.zeros((n, ko // 2), **u8),
+            torch.zeros(abi.sf_bytes(n, kn, abi.MG_OPERAND_B), **u8), torch.zeros(abi.sf_bytes(n, ks, abi.MG_OPERAND_B), **u8),
+            torch.zeros(abi.sf_bytes(n, ko, abi.MG_OPERAND_B), **u8)]
+
+
+def test_fused_linear_refuses_bad_weights_before_any_launch(no_launch):
+    import torch
+    abi = no_launch
+    m, n, kn, ks, ko = 8, 64, 128, 64, 32
+    k = kn + ks + ko
+    x = torch.zeros((m, k), dtype=torch.bfloat16)
+    idx = torch.arange(k, dtype=torch.int16)
+    good = _weights(abi, n, kn, ks, ko)
+    # a well-formed call gets as far as the launch
+    with pytest.raises(AssertionError, match="mg_fused_norm_linear reached"):
+        abi.fused_linear(x, idx, *good, kn, ks, ko)
+    cases = {
+        "wrong dtype": (0, good[0].to(torch.int8)),
+        "too few rows in a segment": (1, good[1][:-1]),
+        "wrong row width": (2, torch.zeros((n, ko // 2 + 16), dtype=torch.uint8)),
+        "not contiguous": (0, torch.zeros((n, kn), dtype=torch.uint8)[:, ::2]),
+        "1-D codes": (0, good[0].reshape(-1)),
+        "short scale buffer": (3, good[3][:-1]),
+        "short scale buffer (last segment)": (5, good[5][:1]),
+        "float scales": (4, good[4].float()),
+    }
+    for what, (pos, t) in cases.items():
+        ops = list(good)
+        ops[pos] = t
+        with pytest.raises(abi.MixedGemmError):
+            abi.fused_linear(x, idx, *ops, kn, ks, ko)
+    # the activations and the index
+    with pytest.raises(abi.MixedGemmError):
+        abi.fused_linear(x[:, :-32].contiguous(), idx, *good, kn, ks, ko)
+    with pytest.raises(abi.MixedGemmError):
+        abi.fused_linear(x, idx[:-1], *good, kn, ks, ko)
+    with pytest.raises(abi.MixedGemmError):
+        abi.fused_linear(x, idx, *good, kn, ks + 16, ko - 16)
+    with pytest.raises(abi.MixedGemmError):
+        abi.fused_linear(x, idx, *good, kn, ks, ko, workspace=torch.zeros(16, dtype=torch.uint8))
+    with pytest.raises(abi.MixedGemmError):
+        abi.fused_linear(x, idx, *good, kn, ks, ko, out=torch.zeros((m, n + 1), dtype=torch.bfloat16))
+
+
+def test_matmul_refuses_short_scale_buffers_before_any_launch(no_launch):
+    import torch
+    abi = no_launch
+    m, n, kn, ks, ko = 8, 64, 128, 64, 32
+    u8 = dict(dtype=torch.uint8)
+    b = _weights(abi, n, kn, ks, ko)
+    a = [torch.zeros((m, kn // 2), **u8), torch.zeros((m, ks // 4 * 3), **u8), torch.zeros((m, ko), **u8),
+         torch.zeros(abi.sf_bytes(m, kn, abi.MG_OPERAND_A), **u8), torch.zeros(abi.sf_bytes(m, ks, abi.MG_OPERAND_A), **u8),
+         torch.zeros(abi.sf_bytes(m, ko, abi.MG_OPERAND_A), **u8)]
+
+    def call(a, b):
+        return abi.matmul(a[0], b[0], a[1], b[1], a[2], b[2], a[3], b[3], a[4], b[4], a[5], b[5])
+
+    with pytest.raises(AssertionError, match="mg_mixed_gemm_ex reached"):
+        call(a, b)
+    for side, pos in (("a", 3), ("a", 4), ("a", 5), ("b", 3), ("b", 4), ("b", 5)):
+        aa, bb = list(a), list(b)
+        (aa if side == "a" else bb)[pos] = (aa if side == "a" else bb)[pos][:-1]
+        with pytest.raises(abi.MixedGemmError, match="bytes, need"):
+            call(aa, bb)
+
+
+def test_the_binding_requires_gpu_tensors(abi):
+    import torch
+    m, n, kn, ks, ko = 8, 64, 128, 64, 32
+    x = torch.zeros((m, kn + ks + ko), dtype=torch.bfloat16)
+    idx = torch.arange(kn + ks + ko, dtype=torch.int16)
+    with pytest.raises(abi.MixedGemmError, match="GPU tensor"):
+        abi.fused_linear(x, idx, *_weights(abi, n, kn, ks, ko), kn, ks, ko)

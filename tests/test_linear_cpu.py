@@ -99,3 +99,28 @@ def test_operators_refuse_cpu_tensors():
     idx = torch.arange(128, dtype=torch.int16)
     with pytest.raises(abi.MixedGemmError):
         torch.ops.mixedgemm_amd.reorder_quantize_x(x, idx, 128, 0, 0)
+
+
+def test_validate_rejects_an_index_outside_the_channels_and_mixed_devices():
+    import pytest
+    import torch
+    from mixedgemm_amd import abi
+    from mixedgemm_amd.linear import PackedWeights
+    n, split = 16, (64, 32, 32)
+    k = sum(split)
+    u8 = dict(dtype=torch.uint8)
+    def make(idx):
+        return PackedWeights(torch.zeros((n, 32), **u8), torch.zeros((n, 16), **u8), torch.zeros((n, 16), **u8),
+                             torch.zeros(abi.sf_bytes(n, 64, abi.MG_OPERAND_B), **u8),
+                             torch.zeros(abi.sf_bytes(n, 32, abi.MG_OPERAND_B), **u8),
+                             torch.zeros(abi.sf_bytes(n, 32, abi.MG_OPERAND_B), **u8), idx, split)
+    make(torch.arange(k, dtype=torch.int16)).validate()
+    for pos, val in ((0, -1), (5, k), (k - 1, 4000)):
+        idx = torch.arange(k, dtype=torch.int16)
+        idx[pos] = val
+        with pytest.raises(ValueError, match="out of range"):
+            make(idx).validate()
+    pw = make(torch.arange(k, dtype=torch.int16))
+    pw.sfwo = pw.sfwo.to("meta")
+    with pytest.raises(ValueError, match="different devices"):
+        pw.validate()

@@ -338,14 +338,15 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
     const int ngroups = ceil_div(rows, R);
     // second LDS buffer: a fixed 16 KB * R behind the first for the 256-lane kernels (see kFixed), else one tile behind
     const int second = K <= 8192 ? 256 * 64 * R : tile;
-    int per_cu = lim.lds_bytes / (second + tile);
+    const int usable = lim.lds_bytes - 1024;   // the kernels' static LDS (row sums of the RMSNorm) stays below 1 KB
+    int per_cu = usable / (second + tile);
     per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
     const int resident = lim.cus * per_cu;
-    const bool stream_groups = ngroups > resident && second + tile <= lim.lds_bytes;
+    const bool stream_groups = ngroups > resident && second + tile <= usable;
     const int grid = stream_groups ? resident : ngroups;
     const int lds = stream_groups ? second + tile : tile;
-    if (lds > lim.lds_bytes) { err = hipErrorInvalidValue; return; }
-    err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), lim.lds_bytes);
+    if (lds > usable) { err = hipErrorInvalidValue; return; }
+    err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), usable);
     if (err != hipSuccess) return;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), (size_t)lds, stream, xb, idx, rows, K,
                        KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream_groups ? tile : 0, gm, eps);

@@ -26,6 +26,7 @@ extern "C" {
 #define MG_ERR_BAD_POINTER 10002 /* null or insufficiently aligned pointer (16 bytes required) */
 #define MG_ERR_BAD_INDEX 10003   /* reorder index entry outside [0, K): mg_check_reorder_index[_host] */
 #define MG_ERR_UNSUPPORTED 10004 /* shape outside what the kernels handle (K > 32736) */
+#define MG_ERR_TOO_LARGE 10005   /* mg_fused_linear_static: the activations do not fit the static scratch memory */
 
 /* Operand selector for mg_sf_bytes(). */
 #define MG_OPERAND_A 0 /* activations: (rows/128 + 1)*128*kseg/32, src/bindings.cpp:91-93 */
@@ -103,6 +104,7 @@ int mg_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, cons
  * GEMMs (src/fp4.cu:164-182) predicate partial tiles themselves and fix their operand layouts.
  */
 #define MG_FLAG_W_TILED 1u
+#define MG_STATIC_SCRATCH_BYTES ((size_t)20 << 20) /* mg_fused_linear_static */
 int mg_mixed_gemm_ex(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                      const uint8_t* ao, const uint8_t* bo,
                      const uint8_t* sfan, const uint8_t* sfbn, const uint8_t* sfas, const uint8_t* sfbs,
@@ -146,6 +148,24 @@ int mg_fused_norm_linear(const void* x_bf16, const void* gamma_bf16, float eps, 
                          int M, int N, int KN, int KS, int KO, unsigned flags,
                          void* d_bf16, void* workspace, size_t workspace_bytes, void* stream);
 size_t mg_fused_workspace_bytes(int M, int KN, int KS, int KO);
+
+/*
+ * mg_fused_linear_ex without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart
+ * in the reference.  The quantized activations go through memory the library owns: a static device array
+ * of MG_STATIC_SCRATCH_BYTES = 20 MiB per GPU, held from the loading of the library until the process
+ * ends.  Problems with mg_fused_workspace_bytes(M, KN, KS, KO) above that size (M = 4096 at K = 4096 and
+ * M = 2048 at K = 14336 fit) are rejected with MG_ERR_TOO_LARGE.  The call allocates and frees nothing;
+ * its first call on a device looks up the array's address on that device (make it outside a capture).
+ * Every call on a GPU uses that GPU's one array: calls that may overlap there (different streams without
+ * an ordering between them, several host threads) race -- order them, or use mg_fused_linear_ex.  Nothing
+ * in the array has to start at zero: a call rewrites every byte its GEMM's results depend on.
+ */
+int mg_fused_linear_static(const void* x_bf16, const int16_t* idx,
+                           const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                           const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo,
+                           int M, int N, int KN, int KS, int KO, unsigned flags,
+                           void* d_bf16, void* stream);
 
 /* Size in bytes of one segment's scale buffer (src/bindings.cpp:91-93, 210-212);
  * never smaller than the interleaved layout spans. */

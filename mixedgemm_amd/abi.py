@@ -24,7 +24,9 @@ SYMBOLS = (
     "mg_fused_linear",
     "mg_fused_workspace_bytes", "mg_sf_bytes", "mg_sf_offset", "mg_device_synchronize", "mg_status_string",
     "mg_calibrate_reorder_index", "mg_calibrate_workspace_bytes", "mg_check_reorder_index", "mg_check_reorder_index_host",
+    "mg_fused_linear_static",
 )
+MG_STATIC_SCRATCH_BYTES = 20 << 20
 
 _lib = None
 
@@ -68,6 +70,8 @@ def lib() -> ctypes.CDLL:
         L.mg_calibrate_workspace_bytes.restype, L.mg_calibrate_workspace_bytes.argtypes = z, [i]
         L.mg_check_reorder_index.restype, L.mg_check_reorder_index.argtypes = i, [p, i, p]
         L.mg_check_reorder_index_host.restype, L.mg_check_reorder_index_host.argtypes = i, [p, i]
+        L.mg_fused_linear_static.restype = i
+        L.mg_fused_linear_static.argtypes = [p] * 8 + [i] * 5 + [u, p, p]
         L.mg_status_string.restype, L.mg_status_string.argtypes = ctypes.c_char_p, [i]
         _lib = L
     return _lib
@@ -305,6 +309,23 @@ def fused_linear(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, wor
                                         MG_FLAG_W_TILED if w_tiled else 0,
                                         _ptr(out), _ptr(workspace), workspace.numel(), _stream(x))
     check(status, "mg_fused_norm_linear")
+    return out
+
+
+def fused_linear_static(x, reorder_index, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko, out, w_tiled=False):
+    """fused_linear through the library's own static scratch memory: the call allocates nothing, so `out`
+    (bf16 [M, N]) is the caller's.  Problems whose quantized activations exceed MG_STATIC_SCRATCH_BYTES are
+    rejected; calls on one GPU must not overlap (they share the scratch memory)."""
+    _check_fused_inputs(x, reorder_index, kn, ks, ko)
+    m = x.shape[0]
+    n = _check_weights(x, bn, bs, bo, sfbn, sfbs, sfbo, kn, ks, ko)
+    _check_out(out, (m, n), torch.bfloat16, "out")
+    if out.device != x.device:
+        raise MixedGemmError("out must be on X's GPU")
+    status = lib().mg_fused_linear_static(_ptr(x), _ptr(reorder_index), _ptr(bn), _ptr(bs), _ptr(bo), _ptr(sfbn),
+                                          _ptr(sfbs), _ptr(sfbo), m, n, kn, ks, ko, MG_FLAG_W_TILED if w_tiled else 0,
+                                          _ptr(out), _stream(x))
+    check(status, "mg_fused_linear_static")
     return out
 
 

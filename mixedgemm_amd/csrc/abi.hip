@@ -52,6 +52,35 @@ int reorder_quantize(const void* x, const int16_t* idx, int rows, int K, int KN,
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
+// Library-owned scratch memory of mg_fused_linear_static: the quantized activations and their scales
+// between the two kernels of a fused call.  One copy per GPU, allocated with the code object and held
+// until the process ends.  `scratch` is a host-side stand-in for the symbol, never a device address:
+// host code uses the per-device pointer scratch_ptr() returns.
+constexpr size_t kScratchBytes = MG_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) uint8_t scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+
+// Device address of `scratch` on the current device, looked up once per device.
+hipError_t scratch_ptr(uint8_t** out) {
+  static std::mutex mu;
+  static uint8_t* table[kMaxDevices] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (table[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (p == nullptr) return hipErrorInvalidSymbol;
+    table[dev] = static_cast<uint8_t*>(p);
+  }
+  *out = table[dev];
+  return hipSuccess;
+}
+
 }  // namespace
 
 extern "C" {
@@ -169,6 +198,19 @@ int mg_fused_linear(const void* x_bf16, const int16_t* idx, const uint8_t* bn, c
                             workspace_bytes, stream);
 }
 
+int mg_fused_linear_static(const void* x_bf16, const int16_t* idx, const uint8_t* bn, const uint8_t* bs, const uint8_t* bo,
+                           const uint8_t* sfbn, const uint8_t* sfbs, const uint8_t* sfbo, int M, int N, int KN, int KS,
+                           int KO, unsigned flags, void* d_bf16, void* stream) {
+  if (int s = check_split(M, KN, KS, KO)) return s;
+  if (N < 0) return MG_ERR_BAD_SHAPE;
+  if (mg_fused_workspace_bytes(M, KN, KS, KO) > kScratchBytes) return MG_ERR_TOO_LARGE;
+  if (M == 0 || N == 0) return MG_OK;
+  uint8_t* ws = nullptr;
+  if (hipError_t e = scratch_ptr(&ws); e != hipSuccess) return (int)e;
+  return mg_fused_norm_linear(x_bf16, nullptr, 0.0f, idx, bn, bs, bo, sfbn, sfbs, sfbo, M, N, KN, KS, KO, flags, d_bf16, ws,
+                              kScratchBytes, stream);
+}
+
 size_t mg_calibrate_workspace_bytes(int K) { return K > 0 ? mg::calibrate_workspace_bytes(K) : 0; }
 
 int mg_calibrate_reorder_index(const void* x_bf16, int M, int K, int16_t* idx, void* workspace, size_t workspace_bytes,
@@ -210,6 +252,7 @@ const char* mg_status_string(int status) {
     case MG_ERR_BAD_POINTER: return "null or misaligned pointer (16-byte alignment required)";
     case MG_ERR_BAD_INDEX: return "reorder index entry out of range";
     case MG_ERR_UNSUPPORTED: return "unsupported shape: K must not exceed 32736";
+    case MG_ERR_TOO_LARGE: return "problem too large for the library's static scratch memory (MG_STATIC_SCRATCH_BYTES)";
     default: return hipGetErrorString(static_cast<hipError_t>(status));
   }
 }

@@ -232,6 +232,8 @@ def test_fused_linear_refuses_bad_weights_before_any_launch(no_launch):
         ops[pos] = t
         with pytest.raises(abi.MixedGemmError):
             abi.fused_linear(x, idx, *ops, kn, ks, ko)
+        with pytest.raises(abi.MixedGemmError):
+            abi.fused_linear_static(x, idx, *ops, kn, ks, ko, out=torch.zeros((m, n), dtype=torch.bfloat16))
     # the activations and the index
     with pytest.raises(abi.MixedGemmError):
         abi.fused_linear(x[:, :-32].contiguous(), idx, *good, kn, ks, ko)
@@ -274,3 +276,18 @@ def test_the_binding_requires_gpu_tensors(abi):
     idx = torch.arange(kn + ks + ko, dtype=torch.int16)
     with pytest.raises(abi.MixedGemmError, match="GPU tensor"):
         abi.fused_linear(x, idx, *_weights(abi, n, kn, ks, ko), kn, ks, ko)
+
+
+def test_static_entry_point_refuses_what_does_not_fit(abi):
+    lib = abi.lib()
+    null = ctypes.c_void_p(0)
+    # 8192 tokens at K = 4096 need 21 MB of quantized activations: more than the 20 MiB the library holds
+    assert abi.fused_workspace_bytes(8192, 2560, 1408, 128) > abi.MG_STATIC_SCRATCH_BYTES
+    assert lib.mg_fused_linear_static(*[null] * 8, 8192, 256, 2560, 1408, 128, 0, null, null) == 10005
+    assert "static scratch" in abi.status_string(10005)
+    # the benchmark configurations fit
+    for m, kn, ks, ko in ((4096, 2560, 1408, 128), (2048, 8960, 4928, 448), (128, 2560, 1408, 128)):
+        assert abi.fused_workspace_bytes(m, kn, ks, ko) <= abi.MG_STATIC_SCRATCH_BYTES
+    # shape errors come first, empty problems succeed without touching the GPU
+    assert lib.mg_fused_linear_static(*[null] * 8, 16, 256, 2560, 1400, 136, 0, null, null) == 10001
+    assert lib.mg_fused_linear_static(*[null] * 8, 0, 256, 2560, 1408, 128, 0, null, null) == 0

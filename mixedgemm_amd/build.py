@@ -37,7 +37,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed FP32 VALU forms are kept out of every kernel
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function",
+    "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
 ]
 
 

@@ -76,6 +76,34 @@ __global__ void __launch_bounds__(256) stream_kernel(const v4u* __restrict__ src
   for (size_t i = t; i < nwrite; i += step) __builtin_nontemporal_store(acc, dst + i);
 }
 
+// The same read stream through global -> LDS copies (global_load_lds_dwordx4): a workgroup of 128 lanes per
+// `row_bytes` (8 KB) piece, pieces blockIdx.x, blockIdx.x + gridDim.x, ..., `depth` pieces requested ahead.
+__global__ void __launch_bounds__(128) stream_lds_kernel(const uint8_t* __restrict__ src, int pieces, int depth,
+                                                         unsigned* __restrict__ sink) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int count = ((int)blockIdx.x < pieces) ? (pieces - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
+  auto request = [&](int i) {
+    const uint8_t* base = src + (size_t)(blockIdx.x + (size_t)i * gridDim.x) * 8192;
+    const unsigned slot = lds0 + (unsigned)(i % depth) * 8192u + wave * 1024u;
+#pragma unroll
+    for (int it = 0; it < 4; ++it)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   : : "v"((unsigned)(it * 128 + tid) * 16u), "s"(base), "s"(slot + it * 2048u) : "memory", "m0");
+  };
+  for (int i = 0; i < depth && i < count; ++i) request(i);
+  unsigned acc = 0;
+  for (int i = 0; i < count; ++i) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_barrier" ::: "memory");
+    acc ^= *reinterpret_cast<const unsigned*>(lds + (i % depth) * 8192 + tid * 64);
+    asm volatile("s_barrier" ::: "memory");
+    if (i + depth < count) request(i + depth);
+  }
+  if (acc == 0x12345678u) sink[0] = acc;
+}
+
 __global__ void __launch_bounds__(1024) empty_kernel(int* __restrict__ sink) {
   if (sink != nullptr && threadIdx.x == 1023 && blockIdx.x == 0x7fffffff) *sink = 0;
 }
@@ -90,6 +118,17 @@ int mgb_stream(const void* src, size_t read_bytes, void* dst, size_t write_bytes
   if (workgroups <= 0 || (read_bytes & 15) || (write_bytes & 15)) return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(mg::stream_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const mg::v4u*>(src), read_bytes / 16, static_cast<mg::v4u*>(dst), write_bytes / 16);
+  return (int)hipGetLastError();
+}
+
+extern "C" __attribute__((visibility("default")))
+int mgb_stream_lds(const void* src, size_t read_bytes, int workgroups, int depth, void* sink, void* stream) {
+  if (workgroups <= 0 || depth <= 0 || depth > 16 || (read_bytes % 8192)) return (int)hipErrorInvalidValue;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mg::stream_lds_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 16 * 8192);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(mg::stream_lds_kernel, dim3(workgroups), dim3(128), depth * 8192, static_cast<hipStream_t>(stream),
+                     static_cast<const uint8_t*>(src), (int)(read_bytes / 8192), depth, static_cast<unsigned*>(sink));
   return (int)hipGetLastError();
 }
 

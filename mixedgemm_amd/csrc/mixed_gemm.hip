@@ -325,6 +325,318 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
   }
 }
 
+// ---------------------------------------------------------------------------
+// Decode kernel: up to 16 tokens, whole 128-wide K steps.
+//
+// The skinny kernel above issues seven loads per K step and wave, five of them for a few bytes each (the
+// token fragment twice, three scale bytes); the address unit handles those as slowly as the two 1 KB weight
+// loads, and with 31 MB to stream in a few microseconds that is what bounds it.  Here everything that is not
+// a weight code goes global -> LDS once per workgroup in 1 KB copies (global_load_lds_dwordx4): the token
+// codes of all three segments (M x 2464 bytes for K = 4096) and, per K step, the 16-byte pieces of the scale
+// atoms that hold the workgroup's rows; the K loop reads them from LDS.  The weight codes go to registers,
+// eight K steps per wave in flight at a time, in two rounds of four.  All
+// requests are inline assembly, so that the waits can count them (requests complete in order).
+//
+// Which features a workgroup owns follows the scale atoms: a 16-byte piece of an atom holds rows c, c + 32,
+// c + 64, c + 96 of a group of 128 (c = row % 32).  Row-major weights: the workgroup of 16 F features takes
+// pieces c0 ... c0 + 4F - 1 of one group, i.e. rows c0 + (i % (4F)) + 32 (i / (4F)) for i = 0 ... 16F - 1 (its
+// results are still runs of four consecutive features).  Tile-major weights: a workgroup takes F of the 1 KB
+// copy blocks of a 256-feature tile (rows j + 32 t + 16 u, t = 0..7, u = 0, 1), whose scales are pieces j and
+// j + 16 of both groups of the tile.  Either way the scales of a step are 64 F contiguous-by-piece bytes.
+//
+// Workgroup = 4 waves; the K steps (over the three segments) are dealt to the waves in contiguous quarters;
+// partial tiles are summed through LDS.
+// ---------------------------------------------------------------------------
+struct DecodeLds {
+  int x0, x1, x2;        // byte offsets of the token codes per segment
+  int sfa0, sfa1, sfa2;  // of the token scale pieces: per step pa pieces of 16 bytes (tokens 0 .. pa - 1)
+  int sfb0, sfb1, sfb2;  // of the weight scale pieces: per step 4 F pieces
+  int partial;           // of the partial sums
+  int total;
+  int pa;                // 8 (up to 8 tokens) or 16
+};
+
+// value of segment seg (0, 1, 2) by masking: a select between struct fields invites the compiler to index a private
+// copy of the struct, which lands in scratch memory
+__device__ __forceinline__ int sel3(int seg, int v0, int v1, int v2) {
+  return (v0 & (seg == 0 ? -1 : 0)) | (v1 & (seg == 1 ? -1 : 0)) | (v2 & (seg == 2 ? -1 : 0));
+}
+__device__ __forceinline__ const uint8_t* sel3p(int seg, const uint8_t* p0, const uint8_t* p1, const uint8_t* p2) {
+  const uint64_t m0 = seg == 0 ? ~0ull : 0ull, m1 = seg == 1 ? ~0ull : 0ull, m2 = seg == 2 ? ~0ull : 0ull;
+  return reinterpret_cast<const uint8_t*>((reinterpret_cast<uint64_t>(p0) & m0) | (reinterpret_cast<uint64_t>(p1) & m1) |
+                                          (reinterpret_cast<uint64_t>(p2) & m2));
+}
+
+__device__ __forceinline__ void dma16_at(const uint8_t* base, unsigned voff, unsigned lds_off) {
+  // base and lds_off are wave-uniform; say so to the compiler
+  const uint64_t bv = reinterpret_cast<uint64_t>(base);
+  // (the builtin returns int: without the casts the low half would be sign-extended over the high half)
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)bv);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(bv >> 32));
+  base = reinterpret_cast<const uint8_t*>(((uint64_t)hi << 32) | lo);
+  lds_off = __builtin_amdgcn_readfirstlane(lds_off);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               : : "v"(voff), "s"(base), "s"(lds_off) : "memory", "m0");
+}
+
+// Copies `bytes` (a multiple of 16) from src to LDS offset dst in units of 1 KB, unit u by wave u % 4; lanes past
+// the end copy the last 16 bytes again (into the padding that rounds every region up to whole units).
+__device__ __forceinline__ void copy_region(const uint8_t* src, int bytes, unsigned dst, int wave, int lane) {
+  const int units = (bytes + 1023) >> 10, chunks = bytes >> 4;
+  for (int u = wave; u < units; u += 4)
+    dma16_at(src, (unsigned)min(u * 64 + lane, chunks - 1) * 16u, dst + (unsigned)u * 1024u);
+}
+
+// Copies P (4, 8 or 16, a power of two) 16-byte pieces per K step of a segment's scale atoms (512 bytes per step)
+// to LDS as [step][piece]; piece_off is this lane's piece (lane % P) as a byte offset inside the atom (and, for
+// pieces of another group of 128 rows, that group's distance).  Units of 1 KB = 64 / P steps, unit u by wave u % 4;
+// steps past the last one copy it again (into the region's padding).
+__device__ __forceinline__ void copy_pieces(const uint8_t* src, int steps, int P, unsigned piece_off, unsigned dst,
+                                            int wave, int lane) {
+  const int per_unit = 64 / P, units = (steps + per_unit - 1) / per_unit;
+  for (int u = wave; u < units; u += 4) {
+    const int q = min(u * per_unit + lane / P, steps - 1);
+    dma16_at(src, (unsigned)q * 512u + piece_off, dst + (unsigned)u * 1024u);
+  }
+}
+
+// 16 bytes global -> registers as an instruction the compiler does not count; use after s_waitcnt + tie()
+__device__ __forceinline__ void load16_uncounted(v4i& dst, const uint8_t* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void tie(v4i& r) { asm volatile("" : "+v"(r)); }
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
+
+template <int F, bool WT>
+__global__ void __launch_bounds__(256)
+mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N, int steps_per_wave, DecodeLds L,
+                         uint16_t* __restrict__ d) {
+  constexpr int S = 4;        // K steps per round
+  constexpr int PB = 4 * F;   // weight scale pieces per step
+  extern __shared__ __align__(16) uint8_t lds[];
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i = lane & 15, g = lane >> 4;
+  // the segments' fields as scalars (selected by masks below, never by indexing)
+  const uint8_t *b4 = s4.b, *b6 = s6.b, *b8 = s8.b;
+  const int nblk4 = s4.nblk, nblk6 = s6.nblk, nblk8 = s8.nblk;
+  const int total = s4.steps + s6.steps + s8.steps;
+  const int t_begin = wave * steps_per_wave, t_end = min(total, t_begin + steps_per_wave);
+  const int rounds = (t_end - t_begin + S - 1) / S;   // may be <= 0 for the last wave
+
+  // ---- the workgroup's rows.  Feature group f, lane row i -> row n[f], its scale piece and its slot in the piece.
+  int n[F], piece[F], slot[F];
+  unsigned sfb_piece_off;   // this lane's piece (lane % PB) of the copies, as a byte offset from the segment's buffer
+  int sfb_katoms_mul;       // ... plus this many times katoms * 512 (the piece's group of 128 rows)
+  if constexpr (WT) {
+    // blocks j0 + f of tile `tile`; pieces ordered [group of 128][u][f]
+    const int tile = (blockIdx.x * F) >> 4, j0 = (blockIdx.x * F) & 15;
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+      const int t = i & 7, u = i >> 3;
+      n[f] = tile * 256 + j0 + f + 32 * t + 16 * u;
+      piece[f] = (t >> 2) * 2 * F + u * F + f;
+      slot[f] = t & 3;
+    }
+    const int pl = lane % PB, pf = pl % F, pu = (pl / F) & 1, pg = pl / (2 * F);
+    sfb_piece_off = (unsigned)(j0 + pf + 16 * pu) * 16u;
+    sfb_katoms_mul = tile * 2 + pg;
+  } else {
+    // pieces c0 ... c0 + PB - 1 of group blockIdx.x / (32 / PB)
+    const int per_group = 32 / PB, group = blockIdx.x / per_group, c0 = (blockIdx.x % per_group) * PB;
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+      const int e = 16 * f + i;   // 0 ... 16 F - 1
+      n[f] = group * 128 + c0 + e % PB + 32 * (e / PB);
+      piece[f] = e % PB;
+      slot[f] = e / PB;
+    }
+    sfb_piece_off = (unsigned)(c0 + lane % PB) * 16u;
+    sfb_katoms_mul = group;
+  }
+
+  // ---- what is not a weight code: requested first, into LDS
+  copy_region(s4.a, M * nblk4 * 16, lds0 + L.x0, wave, lane);
+  copy_region(s6.a, M * nblk6 * 24, lds0 + L.x1, wave, lane);
+  copy_region(s8.a, M * nblk8 * 32, lds0 + L.x2, wave, lane);
+  {
+    const unsigned pa_off = (unsigned)(lane % L.pa) * 16u;   // token scale pieces 0 ... pa - 1 of the first group of rows
+    if (s4.steps) copy_pieces(s4.sfa, s4.steps, L.pa, pa_off, lds0 + L.sfa0, wave, lane);
+    if (s6.steps) copy_pieces(s6.sfa, s6.steps, L.pa, pa_off, lds0 + L.sfa1, wave, lane);
+    if (s8.steps) copy_pieces(s8.sfa, s8.steps, L.pa, pa_off, lds0 + L.sfa2, wave, lane);
+    if (s4.steps) copy_pieces(s4.sfb, s4.steps, PB, sfb_piece_off + (unsigned)(sfb_katoms_mul * s4.steps) * 512u, lds0 + L.sfb0, wave, lane);
+    if (s6.steps) copy_pieces(s6.sfb, s6.steps, PB, sfb_piece_off + (unsigned)(sfb_katoms_mul * s6.steps) * 512u, lds0 + L.sfb1, wave, lane);
+    if (s8.steps) copy_pieces(s8.sfb, s8.steps, PB, sfb_piece_off + (unsigned)(sfb_katoms_mul * s8.steps) * 512u, lds0 + L.sfb2, wave, lane);
+  }
+
+  // ---- weight codes: per lane 16 bytes per step and feature group (row n[f], block g of the step)
+  int nc[F];
+#pragma unroll
+  for (int f = 0; f < F; ++f) nc[f] = min(n[f], N - 1);   // clamped rows: every load is in bounds
+  v4i wq[2][S][F];
+  auto request_round = [&](int r, auto buf_c) {
+    constexpr int B = decltype(buf_c)::value;
+#pragma unroll
+    for (int k = 0; k < S; ++k) {
+      const int t = min(t_begin + r * S + k, total - 1);
+      const int seg = t < s4.steps ? 0 : (t < s4.steps + s6.steps ? 1 : 2);
+      const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
+      const uint8_t* pb = sel3p(seg, b4, b6, b8);
+      const int nblk = sel3(seg, nblk4, nblk6, nblk8);
+#pragma unroll
+      for (int f = 0; f < F; ++f) {
+        const uint8_t* p;
+        if constexpr (WT) {
+          // 16 KB per (256-feature tile, step), the block's 1 KB in it, lane quad i, piece g
+          const int bx = blockIdx.x * F + f;
+          p = pb + ((((size_t)(bx >> 4) * (nblk >> 2) + q) * 16 + (bx & 15)) * 1024 + i * 64 + g * 16);
+        } else {
+          p = pb + (size_t)nc[f] * nblk * 16 + q * 64 + g * 16;
+        }
+        load16_uncounted(wq[B][k][f], p);
+      }
+    }
+  };
+  if (rounds > 0) request_round(0, std::integral_constant<int, 0>{});
+
+  // ---- the copies are older than the weight requests: they are done when only those are in flight
+  if (rounds > 0) wait_vmcnt<S * F>();
+  else wait_vmcnt<0>();
+  asm volatile("s_barrier" ::: "memory");
+
+  v4f acc[F];
+#pragma unroll
+  for (int f = 0; f < F; ++f) acc[f] = v4f{0.f, 0.f, 0.f, 0.f};
+  const int mc = min(i, M - 1);   // token of this lane (tokens past M: the last one again, never stored)
+  const int pa16 = L.pa * 16;
+
+  auto compute_round = [&](int r, auto buf_c) {
+    constexpr int B = decltype(buf_c)::value;
+#pragma unroll
+    for (int k = 0; k < S; ++k) {
+      const int t = t_begin + r * S + k;
+      if (t < t_end) {   // wave-uniform
+        const int seg = t < s4.steps ? 0 : (t < s4.steps + s6.steps ? 1 : 2);
+        const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
+        const uint8_t* sfa_l = lds + sel3(seg, L.sfa0, L.sfa1, L.sfa2) + q * pa16;
+        const uint8_t* sfb_l = lds + sel3(seg, L.sfb0, L.sfb1, L.sfb2) + q * (PB * 16);
+        const int s_x = sfa_l[mc * 16 + g];
+        v8i wf[F];
+        int s_w[F];
+#pragma unroll
+        for (int f = 0; f < F; ++f) {
+          s_w[f] = sfb_l[piece[f] * 16 + slot[f] * 4 + g];
+          const v4i w4 = wq[B][k][f];
+          wf[f] = v8i{w4[0], w4[1], w4[2], w4[3], 0, 0, 0, 0};
+        }
+        if (seg == 0) {
+          const v4i a4 = *reinterpret_cast<const v4i*>(lds + L.x0 + mc * (nblk4 * 16) + q * 64 + g * 16);
+          const v8i xf = {a4[0], a4[1], a4[2], a4[3], 0, 0, 0, 0};
+#pragma unroll
+          for (int f = 0; f < F; ++f) acc[f] = decode_mfma<kFmtE2M1>(wf[f], xf, acc[f], s_w[f], s_x);
+        } else if (seg == 1) {
+          const v2i* p = reinterpret_cast<const v2i*>(lds + L.x1 + mc * (nblk6 * 24) + q * 96 + g * 24);
+          const v2i a = p[0], b = p[1], c = p[2];
+          const v8i xf = {a[0], a[1], b[0], b[1], c[0], c[1], 0, 0};
+#pragma unroll
+          for (int f = 0; f < F; ++f) acc[f] = decode_mfma<kFmtE3M2>(wf[f], xf, acc[f], s_w[f], s_x);
+        } else {
+          const uint8_t* p = lds + L.x2 + mc * (nblk8 * 32) + q * 128 + g * 16;
+          const v4i a4 = *reinterpret_cast<const v4i*>(p), b4v = *reinterpret_cast<const v4i*>(p + 64);
+          const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4v[0], b4v[1], b4v[2], b4v[3]};
+#pragma unroll
+          for (int f = 0; f < F; ++f) acc[f] = decode_mfma<kFmtE4M3>(wf[f], xf, acc[f], s_w[f], s_x);
+        }
+      }
+    }
+  };
+  // the registers of a round are tied to the wait that precedes their use
+  auto settle = [&](auto buf_c, auto n_c) {
+    constexpr int B = decltype(buf_c)::value;
+    constexpr int NW = decltype(n_c)::value;
+    wait_vmcnt<NW>();
+#pragma unroll
+    for (int k = 0; k < S; ++k)
+#pragma unroll
+      for (int f = 0; f < F; ++f) tie(wq[B][k][f]);
+  };
+  // Two rounds per iteration, both requested before the first is used; nothing is in flight across the loop edge
+  // (a register that an uncounted load is still to fill must not be moved by the compiler, which a value carried
+  // around a loop may be).  Round 0 is in flight already.
+  for (int r = 0; r < rounds; r += 2) {
+    if (r > 0) request_round(r, std::integral_constant<int, 0>{});
+    if (r + 1 < rounds) {
+      request_round(r + 1, std::integral_constant<int, 1>{});
+      settle(std::integral_constant<int, 0>{}, std::integral_constant<int, S * F>{});
+    } else {
+      settle(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+    }
+    compute_round(r, std::integral_constant<int, 0>{});
+    if (r + 1 < rounds) {
+      settle(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+      compute_round(r + 1, std::integral_constant<int, 1>{});
+    }
+  }
+
+  // ---- sum the four waves' partial tiles (D^T: lane holds token lane % 16, feature slots 4 * (lane / 16) + v of a group)
+  float* partial = reinterpret_cast<float*>(lds + L.partial);
+#pragma unroll
+  for (int f = 0; f < F; ++f) *reinterpret_cast<v4f*>(partial + ((wave * F + f) * 64 + lane) * 4) = acc[f];
+  __syncthreads();
+#pragma unroll
+  for (int f = 0; f < F; ++f) {
+    if ((f & 3) != wave) continue;
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) sum += *reinterpret_cast<const v4f*>(partial + ((w * F + f) * 64 + lane) * 4);
+    if (i < M) {
+      uint16_t h[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) h[v] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
+      if constexpr (WT) {
+        // feature slot e = 4 g + v of the block is row j + 32 (e % 8) + 16 (e / 8) of the tile
+        const int bx = blockIdx.x * F + f, row0 = (bx >> 4) * 256 + (bx & 15);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int e = 4 * g + v, row = row0 + 32 * (e & 7) + 16 * (e >> 3);
+          if (row < N) d[(size_t)i * N + row] = h[v];
+        }
+      } else {
+        // feature slots 4 g ... 4 g + 3 of the group are four consecutive rows
+        const int per_group = 32 / PB, group = blockIdx.x / per_group, c0 = (blockIdx.x % per_group) * PB;
+        const int e = 16 * f + 4 * g;
+        const int nn = group * 128 + c0 + e % PB + 32 * (e / PB);
+        uint16_t* dst = d + (size_t)i * N + nn;
+        if (nn + 3 < N && (N & 3) == 0) {
+          *reinterpret_cast<v2u*>(dst) = v2u{(unsigned)h[0] | ((unsigned)h[1] << 16), (unsigned)h[2] | ((unsigned)h[3] << 16)};
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (nn + v < N) dst[v] = h[v];
+        }
+      }
+    }
+  }
+}
+
+static int round_up_1k(int v) { return (v + 1023) & ~1023; }
+
+// The decode kernel takes: up to 16 tokens, whole 128-wide steps in every segment, and an LDS image of at most
+// 76 KB (two workgroups per CU).
+static bool decode_lds_plan(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int F, DecodeLds* L) {
+  int pos = 0;
+  auto take = [&](int bytes) { const int at = pos; pos += round_up_1k(bytes); return at; };
+  L->pa = M <= 8 ? 8 : 16;
+  L->x0 = take(M * d4.nblk * 16); L->x1 = take(M * d6.nblk * 24); L->x2 = take(M * d8.nblk * 32);
+  L->sfa0 = take(d4.steps * L->pa * 16); L->sfa1 = take(d6.steps * L->pa * 16); L->sfa2 = take(d8.steps * L->pa * 16);
+  L->sfb0 = take(d4.steps * F * 64); L->sfb1 = take(d6.steps * F * 64); L->sfb2 = take(d8.steps * F * 64);
+  L->partial = pos;
+  pos += 4 * F * 1024;
+  L->total = pos;
+  return pos <= 76 * 1024;
+}
+
 // Feature groups of 16 per workgroup of the skinny kernel.
 static int skinny_feature_groups(int rows, int N) {
   const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
@@ -334,6 +646,23 @@ static int skinny_feature_groups(int rows, int N) {
 hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int N,
                          bool w_tiled, uint16_t* d, hipStream_t stream) {
   const int rows = M;
+  // decode: the kernel that stages everything but the weight codes in LDS
+  if (M <= 16 && ((d4.nblk | d6.nblk | d8.nblk) & 3) == 0) {
+    const int f = skinny_feature_groups(rows, N);
+    DecodeLds L;
+    if (decode_lds_plan(d4, d6, d8, M, f, &L)) {
+      const int spw = (d4.steps + d6.steps + d8.steps + 3) / 4;
+      // row-major: per group of 128 rows 8 / F workgroups (the last group whole, rows past N clamped and not stored)
+      const dim3 grid(w_tiled ? ceil_div(N, 16 * f) : ceil_div(N, 128) * (8 / f));
+      typedef void (*kernel_t)(DecodeSeg, DecodeSeg, DecodeSeg, int, int, int, DecodeLds, uint16_t*);
+      const kernel_t kernels[2][2] = {{mixed_gemm_decode_kernel<1, false>, mixed_gemm_decode_kernel<2, false>},
+                                      {mixed_gemm_decode_kernel<1, true>, mixed_gemm_decode_kernel<2, true>}};
+      const kernel_t kernel = kernels[w_tiled ? 1 : 0][f - 1];
+      if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), 76 * 1024); e != hipSuccess) return e;
+      hipLaunchKernelGGL(kernel, grid, dim3(256), (size_t)L.total, stream, d4, d6, d8, M, N, spw, L, d);
+      return hipGetLastError();
+    }
+  }
   const int steps_per_wave = (d4.steps + d6.steps + d8.steps + 3) / 4;
   const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
   // two feature groups per workgroup for 17-64 tokens: each activation fragment then serves 32 features

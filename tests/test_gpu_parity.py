@@ -186,6 +186,34 @@ GEMM_SHAPES = [
 ]
 
 
+# decode kernel (up to 16 tokens, whole 128-wide steps): one and two feature groups per workgroup, ragged N inside
+# and across groups of 128 rows, an empty segment, a single token, K beyond one round of steps per wave
+DECODE_SHAPES = [
+    (8, 14336, 2560, 1408, 128), (1, 4096, 2560, 1408, 128), (16, 512, 384, 256, 128), (7, 200, 128, 128, 128),
+    (8, 8200, 256, 128, 0), (3, 1000, 2560, 1408, 128), (12, 136, 0, 384, 128), (8, 12288, 1280, 0, 256),
+    (2, 9000, 4096, 2048, 512), (16, 8192, 128, 0, 0),
+]
+
+
+@pytest.mark.parametrize("m,n,kn,ks,ko", DECODE_SHAPES)
+@pytest.mark.parametrize("tiled", [False, True])
+def test_decode_kernel_matches_oracle(abi, m, n, kn, ks, ko, tiled):
+    k = kn + ks + ko
+    _say("decode", m, n, kn, ks, ko, "tiled" if tiled else "row-major")
+    if tiled and not abi.weights_tileable(n, kn, ks, ko):
+        pytest.skip("shape cannot be tiled")
+    x = H.make_activations(m, k, 17 + m + n, n_out=max(1, k // 32))
+    w = H.make_weights(n, k, 19 + m + n)
+    idx = H.absmax_sort_index(x)
+    qx, qw = _oracle_operands(x, w, idx, kn, ks, ko)
+    a, b = _to_dev(qx), _to_dev(qw)
+    if tiled:
+        b = list(abi.tile_weights(*b[:3])) + b[3:]
+    d = abi.matmul(a[0], b[0], a[1], b[1], a[2], b[2], a[3], b[3], a[4], b[4], a[5], b[5], w_tiled=tiled)
+    torch.cuda.synchronize()
+    _check_gemm(d, qx, qw, f"decode {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("m,n,kn,ks,ko", GEMM_SHAPES)
 def test_mixed_gemm_matches_oracle(abi, m, n, kn, ks, ko):
     k = kn + ks + ko

@@ -982,7 +982,7 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO);
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
-                                 int M, int m_store, int a_rows, int N, int KN, int KS, int KO, bool w_tiled, void* d,
+                                 int m_store, int a_rows, int N, int KN, int KS, int KO, bool w_tiled, void* d,
                                  hipStream_t stream);
 
 // Rough launch times in microseconds (measured on MI355X, K = 4096: a 128-wide stage takes ~1.05 us
@@ -1013,8 +1013,8 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
   // a_rows (lanes that would are pointed at the last readable row)
   if (mixed_gemm_256_supported(m_pad, N, KN, KS, KO) &&
       (M >= 256 || pipelined_us(m_pad, N, steps) < skinny_us(M, N, steps)))
-    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, m_pad, M, a_rows, N, KN, KS,
-                                 KO, w_tiled, d, stream);
+    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, a_rows, N, KN, KS, KO,
+                                 w_tiled, d, stream);
   const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
   const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
   const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};

@@ -377,10 +377,10 @@ __device__ __forceinline__ v8i widen(v6i v) { return __builtin_shufflevector(v, 
 __device__ __forceinline__ v8i widen(v8i v) { return v; }
 
 // Fragments of one 64-wide K half of a stage: 4 feature tiles, 4 token tiles.
-template <int FMT>
+template <int FMT, int TM>
 struct HalfFrags {
   v4i w[4];
-  typename Fmt<FMT>::xfrag x[4];
+  typename Fmt<FMT>::xfrag x[TM];
 };
 
 // Per-lane LDS addresses of a wave's fragments in stage buffer 0.
@@ -389,25 +389,27 @@ struct WeightPtrs {
   const uint8_t* sw;   // scale dwords of the 4 feature tiles
   const uint8_t* sx;   // scale dwords of the 4 token tiles
 
-  __device__ __forceinline__ WeightPtrs(const uint8_t* lds, const Ctx& c) {
+  // tm: token tiles of 32 per wave (4: a wave's tokens are one scale atom of 128 rows; 2: both halves share one)
+  __device__ __forceinline__ WeightPtrs(const uint8_t* lds, const Ctx& c, int tm) {
     const int i = c.lane & 31, g = c.lane >> 5;
     w = lds + kWOff + (i & 15) * kBlk + (i >> 4) * 512 + c.wn * 256 + g * 16;
     sw = lds + kSOff + c.wn * 512 + i * 16;
-    sx = lds + kSOff + 1024 + c.wm * 512 + i * 16;
+    sx = lds + kSOff + 1024 + (tm == 4 ? c.wm * 512 : 0) + i * 16;
   }
 };
 
-template <int FMT>
+template <int FMT, int TM>
 struct TokenPtrs {
   const uint8_t* x;
 
+  // the wave's token tiles are tiles TM * wm ... TM * wm + TM - 1 of the workgroup's
   __device__ __forceinline__ TokenPtrs(const uint8_t* lds, const Ctx& c) {
     const int i = c.lane & 31, g = c.lane >> 5;
     if constexpr (FMT == kFmtE3M2) {
       // row 32*rt + i: block i%8, row slot 4*rt + i/8, fragment 2h+g of 24 bytes
-      x = lds + kXOff + (i & 7) * kBlk6 + (16 * c.wm + (i >> 3)) * 96 + g * 24;
+      x = lds + kXOff + (i & 7) * kBlk6 + (4 * TM * c.wm + (i >> 3)) * 96 + g * 24;
     } else {
-      x = lds + kXOff + (i & 15) * kBlk + (i >> 4) * 512 + c.wm * 256 + g * 16;
+      x = lds + kXOff + (i & 15) * kBlk + (i >> 4) * 512 + c.wm * (64 * TM) + g * 16;
     }
   }
 };
@@ -415,9 +417,9 @@ struct TokenPtrs {
 // Reads of the fragments of K half H of one stage, one fragment per call so that they can be
 // spread between MFMAs: R = 0..3 weight tile R, 4..7 token tile R-4, 8 / 9 the scale dwords of
 // the feature / token tiles (only when SC).
-template <int FMT, int H, bool SC>
+template <int FMT, int H, bool SC, int TM>
 struct FragReader {
-  HalfFrags<FMT>& f;
+  HalfFrags<FMT, TM>& f;
   v4i& sw;
   v4i& sx;
   const uint8_t* pw;
@@ -426,14 +428,14 @@ struct FragReader {
   const uint8_t* psx;
   bool on;   // wave-uniform
 
-  static constexpr int kReads = SC ? 10 : 8;
+  static constexpr int kReads = SC ? 6 + TM : 4 + TM;
 
   template <int R>
   __device__ __forceinline__ void read() const {
     if (!on) return;
     if constexpr (R < 4) {
       f.w[R] = *reinterpret_cast<const v4i*>(pw + R * 64 + H * 32);
-    } else if constexpr (R < 8) {
+    } else if constexpr (R < 4 + TM) {
       constexpr int t = R - 4;
       if constexpr (FMT == kFmtE2M1) {
         f.x[t] = *reinterpret_cast<const v4i*>(px + t * 64 + H * 32);
@@ -447,32 +449,37 @@ struct FragReader {
         const v4i b = *reinterpret_cast<const v4i*>(p + 32);   // K [32+16g, 32+16g+16)
         f.x[t] = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
       }
-    } else if constexpr (SC && R == 8) {
+    } else if constexpr (SC && R == 4 + TM) {
       sw = *reinterpret_cast<const v4i*>(psw);
-    } else if constexpr (SC && R == 9) {
+    } else if constexpr (SC && R == 5 + TM) {
       sx = *reinterpret_cast<const v4i*>(psx);
     }
   }
 };
 
-template <int FMT, int H, bool SC, int R = 0>
-__device__ __forceinline__ void read_all(const FragReader<FMT, H, SC>& rd) {
-  if constexpr (R < FragReader<FMT, H, SC>::kReads) {
+template <int R = 0, int FMT, int H, bool SC, int TM>
+__device__ __forceinline__ void read_all(const FragReader<FMT, H, SC, TM>& rd) {
+  if constexpr (R < FragReader<FMT, H, SC, TM>::kReads) {
     rd.template read<R>();
-    read_all<FMT, H, SC, R + 1>(rd);
+    read_all<R + 1>(rd);
   }
 }
 
+template <int TM>
 struct Scales {
-  int w[4], x[4];   // scale dwords of the 4 feature / 4 token tiles, shifted so that byte 0 / 2 is block g / 2+g
+  int w[4], x[TM];   // scale dwords of the 4 feature / TM token tiles, shifted so that byte 0 / 2 is block g / 2+g
 };
 
-__device__ __forceinline__ void shift_scales(Scales& sc, v4i sw, v4i sx, int lane) {
+// sx holds the dwords of the four token tiles of a scale atom; with TM == 2 the wave's are 2 * wm and 2 * wm + 1
+template <int TM>
+__device__ __forceinline__ void shift_scales(Scales<TM>& sc, v4i sw, v4i sx, int lane, int wm) {
   const int g8 = (lane >> 5) * 8;
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    sc.w[t] = (int)((unsigned)sw[t] >> g8);
-    sc.x[t] = (int)((unsigned)sx[t] >> g8);
+  for (int t = 0; t < 4; ++t) sc.w[t] = (int)((unsigned)sw[t] >> g8);
+#pragma unroll
+  for (int t = 0; t < TM; ++t) {
+    const int v = TM == 4 ? sx[t] : (wm ? sx[2 + t] : sx[t]);
+    sc.x[t] = (int)((unsigned)v >> g8);
   }
 }
 
@@ -493,16 +500,17 @@ constexpr int next_slot(int k) { return (k >= 4 + Fmt<FMT>::x_copies && k < 12) 
 // MFMAs stuck behind) and the copy slots [K0, K1) of one stage, one after every second MFMA.
 // LEAN: slots of `lc` (a stage of format CF, skipped when !on) into the buffer at byte offset boff;
 // otherwise slots of the run-time plan `gc`.
-template <int FMT, int H, bool LEAN, int CF, int M0, int K0, int K1, class Reader, bool WT>
-__device__ __forceinline__ void mfma_half(v16f (&acc)[4][4], const HalfFrags<FMT>& f, const Scales& sc, const Reader& rd,
+template <int FMT, int H, bool LEAN, int CF, int M0, int K0, int K1, class Reader, bool WT, int TM>
+__device__ __forceinline__ void mfma_half(v16f (&acc)[4][TM], const HalfFrags<FMT, TM>& f, const Scales<TM>& sc, const Reader& rd,
                                           const LeanCopy<CF, WT>& lc, bool on, unsigned boff, const GenericCopy& gc,
                                           const LaneOffsets& lo, int wave) {
-  if constexpr (M0 < 16) {
-    constexpr int tn = M0 / 4, tm = M0 % 4;
+  if constexpr (M0 < 4 * TM) {
+    constexpr int tn = M0 / TM, tm = M0 % TM;
     mfma_one<FMT, H>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
     if constexpr (M0 < Reader::kReads) rd.template read<M0>();
     constexpr int KS = LEAN ? (CF == kFmtNone ? K1 : next_slot<CF>(K0)) : K0;
-    if constexpr ((M0 & 1) == 1 && KS < K1) {
+    // a copy slot after every second MFMA of 16, after every one of 8
+    if constexpr ((TM == 2 || (M0 & 1) == 1) && KS < K1) {
       if constexpr (LEAN) {
         if (on) lc.template issue<KS>(boff);
       } else {
@@ -539,18 +547,18 @@ struct Ring {
 // (of stage q+3, format CE) from `lce` when early_on; MID says what happens to `lce` between the
 // halves: 1 = advance by one stage, 2 = set up for stage q+3 (first stage of its segment).
 // !LEAN: both from the run-time plan `gc`.  next_on: there is a stage q+1.
-template <int FMT, int FR, bool LEAN, int CL, int CE, int MID, bool WT>
-__device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a, HalfFrags<FR>& a_next, Scales& sc,
+template <int FMT, int FR, bool LEAN, int CL, int CE, int MID, bool WT, int TM>
+__device__ __forceinline__ void stage_body(v16f (&acc)[4][TM], HalfFrags<FMT, TM>& a, HalfFrags<FR, TM>& a_next, Scales<TM>& sc,
                                            const LeanCopy<CL, WT>& lcl, bool late_on, LeanCopy<CE, WT>& lce, bool early_on,
                                            GenericCopy& gc, const LaneOffsets& lo, const Plan& plan, int q,
-                                           bool next_on, const Ring& ring, const WeightPtrs& wp, const TokenPtrs<FMT>& xp,
-                                           const TokenPtrs<FR>& xpn, const Ctx& c) {
-  HalfFrags<FMT> b;
-  HalfFrags<FR> nx;
+                                           bool next_on, const Ring& ring, const WeightPtrs& wp, const TokenPtrs<FMT, TM>& xp,
+                                           const TokenPtrs<FR, TM>& xpn, const Ctx& c) {
+  HalfFrags<FMT, TM> b;
+  HalfFrags<FR, TM> nx;
   v4i sw = {0, 0, 0, 0}, sx = {0, 0, 0, 0};
   wait_lds_reads();   // nothing is outstanding here; tells the compiler so (it cannot see it across the loop edge)
   // first half; reads the second half's fragments; the remaining copies of stage q+2 go to the last buffer
-  const FragReader<FMT, 1, false> rd_b{b, sw, sx, wp.w + ring.cur, xp.x + ring.cur, nullptr, nullptr, true};
+  const FragReader<FMT, 1, false, TM> rd_b{b, sw, sx, wp.w + ring.cur, xp.x + ring.cur, nullptr, nullptr, true};
   mfma_half<FMT, 0, LEAN, CL, 0, kSplit, kCopySlots>(acc, a, sc, rd_b, lcl, late_on, ring.lst, gc, lo, c.wave);
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
@@ -570,12 +578,12 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
   }
   // second half; reads the first half and the scales of stage q+1; the first copies of stage q+3
   // go to the buffer this stage just released
-  const FragReader<FR, 0, true> rd_n{nx, sw, sx, wp.w + ring.nxt, xpn.x + ring.nxt, wp.sw + ring.nxt, wp.sx + ring.nxt,
+  const FragReader<FR, 0, true, TM> rd_n{nx, sw, sx, wp.w + ring.nxt, xpn.x + ring.nxt, wp.sw + ring.nxt, wp.sx + ring.nxt,
                                      next_on};
   mfma_half<FMT, 1, LEAN, CE, 0, 0, kSplit>(acc, b, sc, rd_n, lce, early_on, ring.cur, gc, lo, c.wave);
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
-  shift_scales(sc, sw, sx, c.lane);
+  shift_scales(sc, sw, sx, c.lane, c.wm);
   if constexpr (FR == FMT) a = nx;
   else a_next = nx;
 }
@@ -589,16 +597,16 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][4], HalfFrags<FMT>& a,
 // `lcn`, which the next segment then continues to use as its `lc`.
 // !REGULAR: `gc` describes stage q0 + 2 (whose first copies are out) on entry and exit; the
 // stages that copy across a segment boundary take the run-time path.
-template <int FMT, int F1, int FR1, bool REGULAR, bool WT>
-__device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a, Scales& sc, HalfFrags<FR1>& a_next,
+template <int FMT, int F1, int FR1, bool REGULAR, bool WT, int TM>
+__device__ __forceinline__ void run_segment(v16f (&acc)[4][TM], HalfFrags<FMT, TM>& a, Scales<TM>& sc, HalfFrags<FR1, TM>& a_next,
                                             LeanCopy<FMT, WT>& lc, LeanCopy<F1, WT>& lcn, GenericCopy& gc, const LaneOffsets& lo,
                                             const Plan& plan, int n, int n1, int q0, const WeightPtrs& wp,
                                             const uint8_t* lds, const Ctx& c) {
-  const TokenPtrs<FMT> xp(lds, c);
-  const TokenPtrs<FR1> xpn(lds, c);
+  const TokenPtrs<FMT, TM> xp(lds, c);
+  const TokenPtrs<FR1, TM> xpn(lds, c);
   Ring ring(q0);
   int ql = 0;
-  HalfFrags<FMT> unused;
+  HalfFrags<FMT, TM> unused;
   if constexpr (REGULAR && F1 != kFmtNone) {
     for (; ql + 3 < n; ++ql) {
       stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, true, lc, true, gc, lo, plan, q0 + ql, true, ring, wp, xp,
@@ -662,8 +670,8 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][4], HalfFrags<FMT>& a
 // segment.  Straight-line code: every load is issued (block index clamped into the segment) and
 // absent blocks are turned into zero codes with scale 2^0 afterwards -- branches around code that
 // touches the accumulator make the register allocator spill it.
-template <int FMT>
-__device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+template <int FMT, int TM>
+__device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][TM], const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                  const uint8_t* __restrict__ sfa, const uint8_t* __restrict__ sfb, int blk,
                                                  bool w_tiled, int tiles_n, const Ctx& c) {
   const int r = blk & 3, q = blk >> 2;
@@ -683,16 +691,20 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
     const bool ok = kb < r;
     const int kbc = min(4 * q + kb, blk - 1);           // a block that exists
     const int kb1 = min(4 * q + 2 * h + 1, blk - 1);    // E4M3: the second block of the half
-    HalfFrags<FMT> f;
-    Scales sc;
+    HalfFrags<FMT, TM> f;
+    Scales<TM> sc;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const unsigned n = c.n0 + min(c.wn * 128 + t * 32 + i, c.cols_avail - 1);   // features past the last one are never stored
-      const unsigned m = c.m0 + min(c.wm * 128 + t * 32 + i, c.rows_avail - 1);   // rows past the last readable one are never stored
       const v4i wv = *reinterpret_cast<const v4i*>(wbase + (size_t)n * wpitch + (size_t)max(kbc - wfirst, 0) * 16);
-      const int sw = sfb[sf_offset(n, kbc, katoms)], sx = sfa[sf_offset(m, kbc, katoms)];
+      const int sw = sfb[sf_offset(n, kbc, katoms)];
       f.w[t] = ok ? wv : z;
       sc.w[t] = ok ? sw : 127;
+    }
+#pragma unroll
+    for (int t = 0; t < TM; ++t) {
+      const unsigned m = c.m0 + min(c.wm * (32 * TM) + t * 32 + i, c.rows_avail - 1);   // rows past the last readable one are never stored
+      const int sx = sfa[sf_offset(m, kbc, katoms)];
       sc.x[t] = ok ? sx : 127;
       const uint8_t* xr = a + (size_t)m * lda;
       if constexpr (FMT == kFmtE2M1) {
@@ -717,7 +729,7 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
 #pragma unroll
     for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
-      for (int tm = 0; tm < 4; ++tm) mfma_one<FMT, 0>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
+      for (int tm = 0; tm < TM; ++tm) mfma_one<FMT, 0>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -725,7 +737,11 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][4], const uint8_
 // REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
 // SEGS: which activation segments the plan has, bit 0 E2M1 (always), bit 1 E3M2, bit 2 E4M3 -- the
 // prefetched fragments pass from a segment to the next one that exists, and their types are fixed here.
-template <bool REGULAR, bool REM, bool WT, int SEGS = 7>
+// TM: token tiles of 32 per wave.  4: the workgroup's tile is 256 features x 256 tokens.  2: 256 x 128, for
+// problems with fewer than 256 whole tiles (every CU still gets a workgroup): same copies (the lanes of token
+// rows 128 ... 255 read the last row again, which costs the address unit next to nothing), same LDS image,
+// half the MFMAs per stage, a copy slot after every MFMA instead of every second one.
+template <bool REGULAR, bool REM, bool WT, int SEGS = 7, int TM = 4>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
@@ -769,23 +785,24 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
       tile_m = (j / per_block) * 8 + (r & 7);
     }
   }
+  constexpr int kTokens = 64 * TM;   // token rows of the workgroup's tile
   c.n0 = tile_n * kT;
-  c.m0 = tile_m * kT;
+  c.m0 = tile_m * kTokens;
   c.total = plan.total;
-  c.rows_avail = min(a_rows - c.m0, kT);
+  c.rows_avail = min(a_rows - c.m0, kTokens);
   c.cols_avail = min(N - c.n0, kT);
   c.lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
 
-  v16f acc[4][4];
+  v16f acc[4][TM];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
+    for (int b = 0; b < TM; ++b)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
 
   const LaneOffsets lo(plan, c);
-  const WeightPtrs wp(lds, c);
+  const WeightPtrs wp(lds, c, TM);
 
   // prologue: stages 0 and 1 and the first copies of stage 2 in flight; wait for stage 0 only
   const int n4 = plan.st0, n6 = plan.st1, n8 = plan.st2;
@@ -802,17 +819,17 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   asm volatile("s_barrier" ::: "memory");
 
   static_assert(SEGS == 7 || (REGULAR && !REM && (SEGS == 1 || SEGS == 3 || SEGS == 5)), "plans with an empty segment");
-  HalfFrags<kFmtE2M1> a4, none4;
-  HalfFrags<kFmtE3M2> a6, none6;
-  HalfFrags<kFmtE4M3> a8, none;
-  Scales sc;
+  HalfFrags<kFmtE2M1, TM> a4, none4;
+  HalfFrags<kFmtE3M2, TM> a6, none6;
+  HalfFrags<kFmtE4M3, TM> a8, none;
+  Scales<TM> sc;
   {
-    const TokenPtrs<kFmtE2M1> xp(lds, c);
+    const TokenPtrs<kFmtE2M1, TM> xp(lds, c);
     v4i sw, sx;
-    const FragReader<kFmtE2M1, 0, true> rd{a4, sw, sx, wp.w, xp.x, wp.sw, wp.sx, true};
+    const FragReader<kFmtE2M1, 0, true, TM> rd{a4, sw, sx, wp.w, xp.x, wp.sw, wp.sx, true};
     read_all(rd);
     wait_lds_reads();
-    shift_scales(sc, sw, sx, c.lane);
+    shift_scales(sc, sw, sx, c.lane, c.wm);
   }
   LeanCopy<kFmtE2M1, WT> l4;
   LeanCopy<kFmtE3M2, WT> l6;
@@ -847,12 +864,12 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   constexpr int kPitch = 256 + 16;   // bytes per token row in LDS
   static_assert(4 * 128 * kPitch <= kBuffers * kStage, "epilogue staging must fit the stage buffers");
   __syncthreads();                   // every wave is done with the last stage's fragments
-  uint8_t* stage = lds + c.wave * 128 * kPitch;
+  uint8_t* stage = lds + c.wave * (32 * TM) * kPitch;
   {
     const int g = c.lane >> 5;
     uint8_t* wr = stage + (c.lane & 31) * kPitch + 8 * g;
 #pragma unroll
-    for (int tm = 0; tm < 4; ++tm)
+    for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
       for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
@@ -866,16 +883,16 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   {
     const int r = c.lane >> 4, cc = c.lane & 15;
     const uint8_t* rd = stage + r * kPitch + cc * 16;
-    uint16_t* out = d + (size_t)(c.m0 + c.wm * 128 + r) * N + c.n0 + c.wn * 128 + cc * 8;
+    uint16_t* out = d + (size_t)(c.m0 + c.wm * (32 * TM) + r) * N + c.n0 + c.wn * 128 + cc * 8;
     // token rows at or past m_store are not written, nor the 8-feature pieces past the layer's last feature
-    const int rows_left = (c.wn * 128 + cc * 8 < c.cols_avail) ? m_store - (c.m0 + c.wm * 128 + r) : 0;
+    const int rows_left = (c.wn * 128 + cc * 8 < c.cols_avail) ? m_store - (c.m0 + c.wm * (32 * TM) + r) : 0;
     // Eight reads in flight, then their eight stores: a read that is waited for before its own store costs a
     // full LDS latency per row (which is what the compiler makes of the predicated form: it sinks each read
     // into its store's block -- hence the separate path for tiles that are stored whole).  Streaming stores: the result is not read again here, and the XCD's L2 is
     // better spent on the operands.
     auto write_rows = [&](auto whole) {
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
+      for (int b = 0; b < TM; ++b) {
         v4u v[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const v4u*>(rd + (b * 8 + j) * 4 * kPitch);
@@ -887,7 +904,7 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
         }
       }
     };
-    if (m_store - c.m0 >= kT && c.cols_avail == kT) write_rows(std::true_type{});   // wave-uniform: the whole tile is stored
+    if (m_store - c.m0 >= kTokens && c.cols_avail == kT) write_rows(std::true_type{});   // wave-uniform: the whole tile is stored
     else write_rows(std::false_type{});
   }
 }
@@ -911,31 +928,52 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
   return false;
 }
 
+// Token rows per workgroup tile for a problem of m_store tokens: 256, or 128 when the 256 x 256 tiles would leave
+// at least half of the CUs without one.  A half tile takes about 0.8 of a whole tile's time (the copies of a stage
+// bound it, not its MFMAs), so halves pay only where they put idle CUs to work: measured, M = 2048 N = 4096
+// K = 14336 (128 whole tiles) 99 -> 84 us, M = 1024 N = 4096 K = 4096 (64) 28 -> 22 us, but 896 whole tiles 145 -> 170 us.
+static int tile_tokens(int m_store, int N) {
+  const long long tiles = (long long)((m_store + kT - 1) / kT) * ((N + kT - 1) / kT);
+  return tiles <= 128 ? 128 : 256;
+}
+
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
-                                 int M, int m_store, int a_rows, int N, int KN, int KS, int KO, bool w_tiled, void* d,
+                                 int m_store, int a_rows, int N, int KN, int KS, int KO, bool w_tiled, void* d,
                                  hipStream_t stream) {
-  // M: whole tiles; rows [m_store, M) are computed but not stored; the activation buffers are read up to row
-  // a_rows - 1 only
-  if (m_store > M || m_store <= M - kT || a_rows < m_store) return hipErrorInvalidValue;
+  // m_store tokens are computed in whole tiles of 256 or 128 token rows; rows past m_store are computed but not
+  // stored; the activation buffers are read up to row a_rows - 1 only
+  if (m_store <= 0 || a_rows < m_store) return hipErrorInvalidValue;
+  const int tokens = tile_tokens(m_store, N);
+  const int M = (m_store + tokens - 1) / tokens * tokens;
   // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
   const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
   const bool rem = (KN | KS | KO) % 128 != 0;
   typedef void (*kernel_t)(Plan, int, int, int, int, uint16_t*);
-  // [tiled][regular][rem]
-  const kernel_t kernels[2][2][2] = {
-      {{mixed_gemm_256_kernel<false, false, false>, mixed_gemm_256_kernel<false, true, false>},
-       {mixed_gemm_256_kernel<true, false, false>, mixed_gemm_256_kernel<true, true, false>}},
-      {{mixed_gemm_256_kernel<false, false, true>, mixed_gemm_256_kernel<false, true, true>},
-       {mixed_gemm_256_kernel<true, false, true>, mixed_gemm_256_kernel<true, true, true>}}};
-  // plans with an empty segment: [tiled][which]; which = 0: E2M1 only, 1: E2M1 + E3M2, 2: E2M1 + E4M3
-  const kernel_t partial[2][3] = {
-      {mixed_gemm_256_kernel<true, false, false, 1>, mixed_gemm_256_kernel<true, false, false, 3>,
-       mixed_gemm_256_kernel<true, false, false, 5>},
-      {mixed_gemm_256_kernel<true, false, true, 1>, mixed_gemm_256_kernel<true, false, true, 3>,
-       mixed_gemm_256_kernel<true, false, true, 5>}};
-  const kernel_t kernel = (KS > 0 && KO > 0) ? kernels[w_tiled][regular][rem] : partial[w_tiled][KS > 0 ? 1 : (KO > 0 ? 2 : 0)];
+  // [half tiles][tiled][regular][rem]
+  const kernel_t kernels[2][2][2][2] = {
+      {{{mixed_gemm_256_kernel<false, false, false>, mixed_gemm_256_kernel<false, true, false>},
+        {mixed_gemm_256_kernel<true, false, false>, mixed_gemm_256_kernel<true, true, false>}},
+       {{mixed_gemm_256_kernel<false, false, true>, mixed_gemm_256_kernel<false, true, true>},
+        {mixed_gemm_256_kernel<true, false, true>, mixed_gemm_256_kernel<true, true, true>}}},
+      {{{mixed_gemm_256_kernel<false, false, false, 7, 2>, mixed_gemm_256_kernel<false, true, false, 7, 2>},
+        {mixed_gemm_256_kernel<true, false, false, 7, 2>, mixed_gemm_256_kernel<true, true, false, 7, 2>}},
+       {{mixed_gemm_256_kernel<false, false, true, 7, 2>, mixed_gemm_256_kernel<false, true, true, 7, 2>},
+        {mixed_gemm_256_kernel<true, false, true, 7, 2>, mixed_gemm_256_kernel<true, true, true, 7, 2>}}}};
+  // plans with an empty segment: [half tiles][tiled][which]; which = 0: E2M1 only, 1: E2M1 + E3M2, 2: E2M1 + E4M3
+  const kernel_t partial[2][2][3] = {
+      {{mixed_gemm_256_kernel<true, false, false, 1>, mixed_gemm_256_kernel<true, false, false, 3>,
+        mixed_gemm_256_kernel<true, false, false, 5>},
+       {mixed_gemm_256_kernel<true, false, true, 1>, mixed_gemm_256_kernel<true, false, true, 3>,
+        mixed_gemm_256_kernel<true, false, true, 5>}},
+      {{mixed_gemm_256_kernel<true, false, false, 1, 2>, mixed_gemm_256_kernel<true, false, false, 3, 2>,
+        mixed_gemm_256_kernel<true, false, false, 5, 2>},
+       {mixed_gemm_256_kernel<true, false, true, 1, 2>, mixed_gemm_256_kernel<true, false, true, 3, 2>,
+        mixed_gemm_256_kernel<true, false, true, 5, 2>}}};
+  const int half = tokens == 128 ? 1 : 0;
+  const kernel_t kernel = (KS > 0 && KO > 0) ? kernels[half][w_tiled][regular][rem]
+                                             : partial[half][w_tiled][KS > 0 ? 1 : (KO > 0 ? 2 : 0)];
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kBuffers * kStage); e != hipSuccess) return e;
   Plan p;
   p.a0 = an; p.a1 = as_; p.a2 = ao;
@@ -947,7 +985,7 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.total = p.st0 + p.st1 + p.st2;
   p.w_tiled = w_tiled ? 1 : 0;
   if (w_tiled && N % kT != 0) return hipErrorInvalidValue;
-  const int tiles_n = (N + kT - 1) / kT, tiles_m = M / kT;
+  const int tiles_n = (N + kT - 1) / kT, tiles_m = M / tokens;
   hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store,
                      a_rows, static_cast<uint16_t*>(d));
   return hipGetLastError();

@@ -590,6 +590,11 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][TM], HalfFrags<FMT, TM
 
 // Runs the n >= 1 stages [q0, q0 + n) of one segment whose format is FMT; the next segment has
 // format F1 (kFmtNone after the last one) and n1 stages; FR1 = F1, or FMT after the last segment.
+// NLAST (REGULAR kernels): how many stages the plan's last segment has -- 1, 2, or 3 for three or
+// more; 0 = not known at compile time (plans of one segment) or, for a segment before the last
+// but one, not needed.  It makes "does the stage that would be copied exist" a compile-time
+// constant in every stage body: a run-time switch around each copy costs a branch per copy, at
+// every branch the wait for the fragment reads just issued, and registers (the kernels spilled).
 // On entry `a` holds the first K half of stage q0 and `sc` its scales; on exit `a_next` holds the
 // first half of stage q0 + n when there is one.
 // REGULAR (every segment but the last has at least 3 stages): `lc` describes the copies of local
@@ -597,7 +602,7 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][TM], HalfFrags<FMT, TM
 // `lcn`, which the next segment then continues to use as its `lc`.
 // !REGULAR: `gc` describes stage q0 + 2 (whose first copies are out) on entry and exit; the
 // stages that copy across a segment boundary take the run-time path.
-template <int FMT, int F1, int FR1, bool REGULAR, bool WT, int TM>
+template <int FMT, int F1, int FR1, bool REGULAR, int NLAST = 0, bool WT, int TM>
 __device__ __forceinline__ void run_segment(v16f (&acc)[4][TM], HalfFrags<FMT, TM>& a, Scales<TM>& sc, HalfFrags<FR1, TM>& a_next,
                                             LeanCopy<FMT, WT>& lc, LeanCopy<F1, WT>& lcn, GenericCopy& gc, const LaneOffsets& lo,
                                             const Plan& plan, int n, int n1, int q0, const WeightPtrs& wp,
@@ -613,16 +618,19 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][TM], HalfFrags<FMT, T
                                               xp, c);
       ring.rotate();
     }
-    stage_body<FMT, FMT, true, FMT, F1, 2>(acc, a, unused, sc, lc, true, lcn, n1 > 0, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+    // the last three stages copy stages 0, 1, 2 of the next segment; only the plan's last segment can have
+    // fewer than three (NLAST = 1, 2)
+    constexpr bool s1 = NLAST != 1, s2 = NLAST != 1 && NLAST != 2;
+    stage_body<FMT, FMT, true, FMT, F1, 2>(acc, a, unused, sc, lc, true, lcn, true, gc, lo, plan, q0 + ql, true, ring, wp, xp,
                                            xp, c);
     ring.rotate();
     ++ql;
-    stage_body<FMT, FMT, true, F1, F1, 1>(acc, a, unused, sc, lcn, n1 > 0, lcn, n1 > 1, gc, lo, plan, q0 + ql, true, ring, wp,
-                                          xp, xp, c);
+    stage_body<FMT, FMT, true, F1, F1, 1>(acc, a, unused, sc, lcn, true, lcn, s1, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+                                          xp, c);
     ring.rotate();
     ++ql;
-    stage_body<FMT, FR1, true, F1, F1, 1>(acc, a, a_next, sc, lcn, n1 > 1, lcn, n1 > 2, gc, lo, plan, q0 + ql, true, ring, wp,
-                                          xp, xpn, c);
+    stage_body<FMT, FR1, true, F1, F1, 1>(acc, a, a_next, sc, lcn, s1, lcn, s2, gc, lo, plan, q0 + ql, true, ring, wp, xp, xpn,
+                                          c);
   } else if constexpr (REGULAR) {
     // last segment: its own stages only, any n >= 1; first the stages whose copies all exist (no run-time
     // switches in the body), then the last three
@@ -631,10 +639,17 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][TM], HalfFrags<FMT, T
                                               xp, c);
       ring.rotate();
     }
-    for (; ql + 1 < n; ++ql) {
-      stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, ql + 2 < n, lc, ql + 3 < n, gc, lo, plan, q0 + ql,
-                                              true, ring, wp, xp, xp, c);
+    if ((NLAST == 0 && n >= 3) || NLAST >= 3) {   // third from last: the last stage's remaining copies
+      stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, true, lc, false, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+                                              xp, c);
       ring.rotate();
+      ++ql;
+    }
+    if ((NLAST == 0 && n >= 2) || NLAST >= 2) {   // second from last: nothing left to copy
+      stage_body<FMT, FMT, true, FMT, FMT, 1>(acc, a, unused, sc, lc, false, lc, false, gc, lo, plan, q0 + ql, true, ring, wp, xp,
+                                              xp, c);
+      ring.rotate();
+      ++ql;
     }
     stage_body<FMT, FMT, true, kFmtNone, kFmtNone, 0>(acc, a, unused, sc, lcn, false, lcn, false, gc, lo, plan, q0 + ql,
                                                       false, ring, wp, xp, xp, c);
@@ -741,7 +756,8 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][TM], const uint8
 // problems with fewer than 256 whole tiles (every CU still gets a workgroup): same copies (the lanes of token
 // rows 128 ... 255 read the last row again, which costs the address unit next to nothing), same LDS image,
 // half the MFMAs per stage, a copy slot after every MFMA instead of every second one.
-template <bool REGULAR, bool REM, bool WT, int SEGS = 7, int TM = 4>
+// NLAST: see run_segment (the launcher picks the instance from the plan).
+template <bool REGULAR, bool REM, bool WT, int SEGS = 7, int TM = 4, int NLAST = 0>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d) {
   extern __shared__ __align__(16) uint8_t lds[];
@@ -838,14 +854,14 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   if constexpr (REGULAR) l4.init(plan, 2, lo, c);
   if constexpr (SEGS == 7) {
     run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
-    run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
-    run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4 + n6, wp, lds, c);
+    run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR, NLAST>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
+    run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR, NLAST>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4 + n6, wp, lds, c);
   } else if constexpr (SEGS == 5) {
-    run_segment<kFmtE2M1, kFmtE4M3, kFmtE4M3, REGULAR>(acc, a4, sc, a8, l4, l8, gc, lo, plan, n4, n8, 0, wp, lds, c);
-    run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4, wp, lds, c);
+    run_segment<kFmtE2M1, kFmtE4M3, kFmtE4M3, REGULAR, NLAST>(acc, a4, sc, a8, l4, l8, gc, lo, plan, n4, n8, 0, wp, lds, c);
+    run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR, NLAST>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4, wp, lds, c);
   } else if constexpr (SEGS == 3) {
-    run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
-    run_segment<kFmtE3M2, kFmtNone, kFmtE3M2, REGULAR>(acc, a6, sc, none6, l6, l0, gc, lo, plan, n6, 0, n4, wp, lds, c);
+    run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR, NLAST>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
+    run_segment<kFmtE3M2, kFmtNone, kFmtE3M2, REGULAR, NLAST>(acc, a6, sc, none6, l6, l0, gc, lo, plan, n6, 0, n4, wp, lds, c);
   } else {
     run_segment<kFmtE2M1, kFmtNone, kFmtE2M1, REGULAR>(acc, a4, sc, none4, l4, l0, gc, lo, plan, n4, 0, 0, wp, lds, c);
   }
@@ -937,6 +953,29 @@ static int tile_tokens(int m_store, int N) {
   return tiles <= 128 ? 128 : 256;
 }
 
+typedef void (*kernel_t)(Plan, int, int, int, int, uint16_t*);
+
+// The kernel for a plan: segs = which activation segments exist (bit 0 E2M1, 1 E3M2, 2 E4M3), nlast = stages of the
+// last one (3 = three or more).  Plans with an empty segment exist in the REGULAR, whole-stage form only.
+template <bool REM, bool WT, int TM>
+static kernel_t select_kernel(bool regular, int segs, int nlast) {
+  if (segs == 7) {
+    if (!regular) return mixed_gemm_256_kernel<false, REM, WT, 7, TM, 0>;
+    return nlast == 1 ? mixed_gemm_256_kernel<true, REM, WT, 7, TM, 1>
+                      : (nlast == 2 ? mixed_gemm_256_kernel<true, REM, WT, 7, TM, 2> : mixed_gemm_256_kernel<true, REM, WT, 7, TM, 3>);
+  }
+  if constexpr (!REM) {
+    if (segs == 1) return mixed_gemm_256_kernel<true, false, WT, 1, TM, 0>;
+    if (segs == 3)
+      return nlast == 1 ? mixed_gemm_256_kernel<true, false, WT, 3, TM, 1>
+                        : (nlast == 2 ? mixed_gemm_256_kernel<true, false, WT, 3, TM, 2> : mixed_gemm_256_kernel<true, false, WT, 3, TM, 3>);
+    if (segs == 5)
+      return nlast == 1 ? mixed_gemm_256_kernel<true, false, WT, 5, TM, 1>
+                        : (nlast == 2 ? mixed_gemm_256_kernel<true, false, WT, 5, TM, 2> : mixed_gemm_256_kernel<true, false, WT, 5, TM, 3>);
+  }
+  return nullptr;
+}
+
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
@@ -950,30 +989,19 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
   const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
   const bool rem = (KN | KS | KO) % 128 != 0;
-  typedef void (*kernel_t)(Plan, int, int, int, int, uint16_t*);
-  // [half tiles][tiled][regular][rem]
-  const kernel_t kernels[2][2][2][2] = {
-      {{{mixed_gemm_256_kernel<false, false, false>, mixed_gemm_256_kernel<false, true, false>},
-        {mixed_gemm_256_kernel<true, false, false>, mixed_gemm_256_kernel<true, true, false>}},
-       {{mixed_gemm_256_kernel<false, false, true>, mixed_gemm_256_kernel<false, true, true>},
-        {mixed_gemm_256_kernel<true, false, true>, mixed_gemm_256_kernel<true, true, true>}}},
-      {{{mixed_gemm_256_kernel<false, false, false, 7, 2>, mixed_gemm_256_kernel<false, true, false, 7, 2>},
-        {mixed_gemm_256_kernel<true, false, false, 7, 2>, mixed_gemm_256_kernel<true, true, false, 7, 2>}},
-       {{mixed_gemm_256_kernel<false, false, true, 7, 2>, mixed_gemm_256_kernel<false, true, true, 7, 2>},
-        {mixed_gemm_256_kernel<true, false, true, 7, 2>, mixed_gemm_256_kernel<true, true, true, 7, 2>}}}};
-  // plans with an empty segment: [half tiles][tiled][which]; which = 0: E2M1 only, 1: E2M1 + E3M2, 2: E2M1 + E4M3
-  const kernel_t partial[2][2][3] = {
-      {{mixed_gemm_256_kernel<true, false, false, 1>, mixed_gemm_256_kernel<true, false, false, 3>,
-        mixed_gemm_256_kernel<true, false, false, 5>},
-       {mixed_gemm_256_kernel<true, false, true, 1>, mixed_gemm_256_kernel<true, false, true, 3>,
-        mixed_gemm_256_kernel<true, false, true, 5>}},
-      {{mixed_gemm_256_kernel<true, false, false, 1, 2>, mixed_gemm_256_kernel<true, false, false, 3, 2>,
-        mixed_gemm_256_kernel<true, false, false, 5, 2>},
-       {mixed_gemm_256_kernel<true, false, true, 1, 2>, mixed_gemm_256_kernel<true, false, true, 3, 2>,
-        mixed_gemm_256_kernel<true, false, true, 5, 2>}}};
   const int half = tokens == 128 ? 1 : 0;
-  const kernel_t kernel = (KS > 0 && KO > 0) ? kernels[half][w_tiled][regular][rem]
-                                             : partial[half][w_tiled][KS > 0 ? 1 : (KO > 0 ? 2 : 0)];
+  const int segs = 1 | (KS > 0 ? 2 : 0) | (KO > 0 ? 4 : 0);
+  const int last_stages = KO > 0 ? KO / 128 : (KS > 0 ? KS / 128 : KN / 128);
+  const int nlast = last_stages >= 3 ? 3 : last_stages;
+  kernel_t kernel = nullptr;
+  if (rem) {
+    if (w_tiled) kernel = half ? select_kernel<true, true, 2>(regular, segs, nlast) : select_kernel<true, true, 4>(regular, segs, nlast);
+    else kernel = half ? select_kernel<true, false, 2>(regular, segs, nlast) : select_kernel<true, false, 4>(regular, segs, nlast);
+  } else {
+    if (w_tiled) kernel = half ? select_kernel<false, true, 2>(regular, segs, nlast) : select_kernel<false, true, 4>(regular, segs, nlast);
+    else kernel = half ? select_kernel<false, false, 2>(regular, segs, nlast) : select_kernel<false, false, 4>(regular, segs, nlast);
+  }
+  if (kernel == nullptr) return hipErrorInvalidValue;
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kBuffers * kStage); e != hipSuccess) return e;
   Plan p;
   p.a0 = an; p.a1 = as_; p.a2 = ao;

@@ -176,7 +176,7 @@ GEMM_SHAPES = [
     (300, 512, 2560, 1408, 128), (257, 256, 384, 384, 384), (767, 256, 448, 416, 224),
     # plans without E3M2 and / or E4M3 activations on the whole-tile kernel (fragments pass to the next segment that exists)
     (256, 256, 512, 0, 0), (512, 512, 128, 0, 0), (300, 256, 384, 0, 128), (256, 512, 1024, 0, 256), (256, 256, 384, 256, 0),
-    (300, 512, 2560, 1536, 0), (1000, 256, 4096, 0, 0),
+    (300, 512, 2560, 1536, 0), (1000, 256, 4096, 0, 0), (256, 256, 512, 0, 384), (256, 256, 384, 128, 0),
     # feature counts that are not whole 256-feature tiles (multiples of 8): the last tile's lanes read the last
     # weight row again and store only the pieces that exist
     (300, 1000, 2560, 1408, 128), (256, 264, 384, 384, 384), (512, 136, 448, 416, 224), (700, 8, 128, 128, 128),
@@ -226,6 +226,35 @@ def test_mixed_gemm_matches_oracle(abi, m, n, kn, ks, ko):
     d = abi.matmul(a[0], b[0], a[1], b[1], a[2], b[2], a[3], b[3], a[4], b[4], a[5], b[5])
     torch.cuda.synchronize()
     _check_gemm(d, qx, qw, f"gemm {m}x{n}x{k}")
+
+
+# More than 128 whole tiles: 256 x 256 tiles (smaller problems run 256 x 128).  One plan per kernel family: all three
+# segments with a last segment of 1, 2 and 3 stages (the kernels are compiled per length of the last segment),
+# segments with a remainder, and the plans with an empty segment.
+BIG_TILE_SHAPES = [
+    (2304, 3840, 384, 384, 128), (2304, 3840, 384, 384, 256), (2304, 3840, 384, 384, 384), (2304, 3840, 448, 416, 224),
+    (2304, 3840, 512, 0, 0), (2304, 3840, 384, 128, 0), (2304, 3840, 384, 256, 0), (2304, 3840, 384, 0, 128),
+    (2304, 3840, 384, 0, 384), (2100, 3848, 384, 384, 128),
+]
+
+
+@pytest.mark.parametrize("m,n,kn,ks,ko", BIG_TILE_SHAPES)
+def test_whole_tile_kernel_with_256_token_tiles(abi, m, n, kn, ks, ko):
+    k = kn + ks + ko
+    _say("gemm, 256 x 256 tiles", m, n, kn, ks, ko)
+    x = H.make_activations(m, k, 41 + m + n, n_out=max(1, k // 32))
+    w = H.make_weights(n, k, 43 + m + n)
+    idx = H.absmax_sort_index(x)
+    qx, qw = _oracle_operands(x, w, idx, kn, ks, ko)
+    a, b = _to_dev(qx), _to_dev(qw)
+    d = abi.matmul(a[0], b[0], a[1], b[1], a[2], b[2], a[3], b[3], a[4], b[4], a[5], b[5])
+    torch.cuda.synchronize()
+    _check_gemm(d, qx, qw, f"gemm {m}x{n}x{k}")
+    if abi.weights_tileable(n, kn, ks, ko):
+        bt = list(abi.tile_weights(*b[:3])) + b[3:]
+        dt = abi.matmul(a[0], bt[0], a[1], bt[1], a[2], bt[2], a[3], bt[3], a[4], bt[4], a[5], bt[5], w_tiled=True)
+        torch.cuda.synchronize()
+        assert torch.equal(d, dt)
 
 
 @pytest.mark.parametrize("seg", ["n", "s", "o"])

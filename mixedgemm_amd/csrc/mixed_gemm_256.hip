@@ -347,6 +347,14 @@ struct LeanCopy<kFmtNone, WT> {
   __device__ __forceinline__ void issue(unsigned) const {}
 };
 
+template <int K0, int K1, int FMT, bool WT>
+__device__ __forceinline__ void issue_range(const LeanCopy<FMT, WT>& lc, unsigned boff) {
+  if constexpr (K0 < K1) {
+    lc.template issue<K0>(boff);
+    issue_range<K0 + 1, K1>(lc, boff);
+  }
+}
+
 // s_waitcnt vmcnt(n) for a run-time, wave-uniform n: the n most recent copies may stay in flight
 __device__ __forceinline__ void wait_copies_but(int n) {
   switch (n) {
@@ -781,9 +789,10 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   c.wn = c.wave & 1;
   c.wm = c.wave >> 1;
-  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give each XCD a
-  // contiguous band of feature tiles, and inside the band walk blocks of 8 token tiles, so that
-  // the ~32 tiles an XCD works on at a time share 4 weight tiles and 8 token tiles.
+  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give each XCD a contiguous band of
+  // feature tiles and walk it feature tile by feature tile inside groups of at most 8 feature tiles, token tile
+  // after token tile: the ~32 tiles an XCD works on at a time are then about as many feature tiles as token tiles
+  // (7 x 4.6 for 56 x 16 tiles), which is what keeps the bytes that pass its L2 lowest.
   const int wg = blockIdx.x, nwg = gridDim.x;
   const int tiles_m = nwg / tiles_n;
   int tile_n = wg / tiles_m, tile_m = wg % tiles_m;
@@ -793,12 +802,15 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
     int tile = (wg & 7) * per_xcd + j;           // feature-major tile index
     tile_n = tile / tiles_m;
     tile_m = tile % tiles_m;
-    if (per_xcd % tiles_m == 0 && (tiles_m & 7) == 0) {
+    if (per_xcd % tiles_m == 0) {
       const int cols = per_xcd / tiles_m;        // feature tiles of the band
-      const int per_block = cols * 8;
-      const int r = j % per_block;
-      tile_n = (wg & 7) * cols + r / 8;
-      tile_m = (j / per_block) * 8 + (r & 7);
+      const int groups = (cols + 7) / 8;
+      if (cols % groups == 0) {
+        const int gw = cols / groups, per_group = gw * tiles_m;
+        const int g = j / per_group, r = j % per_group;
+        tile_n = (wg & 7) * cols + g * gw + r % gw;
+        tile_m = r / gw;
+      }
     }
   }
   constexpr int kTokens = 64 * TM;   // token rows of the workgroup's tile
@@ -809,6 +821,41 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   c.cols_avail = min(N - c.n0, kT);
   c.lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
 
+  const LaneOffsets lo(plan, c);
+  const WeightPtrs wp(lds, c, TM);
+
+  // prologue: stages 0 and 1 and the first copies of stage 2 in flight; wait for stage 0 only.  The copies go out
+  // before anything else that can wait (the accumulators are cleared while they are in flight); in REGULAR kernels
+  // the first three stages are E2M1 stages, or do not exist, and take the compile-time form of the copies.
+  const int n4 = plan.st0, n6 = plan.st1, n8 = plan.st2;
+  GenericCopy gc;
+  LeanCopy<kFmtE2M1, WT> l4;
+  int in_flight;   // copies that may stay in flight while stage 0 is awaited
+  if constexpr (REGULAR) {
+    l4.init(plan, 0, lo, c);
+    issue_range<0, kCopySlots>(l4, 0);
+    in_flight = 0;
+    if (plan.total > 1) {
+      l4.advance();
+      issue_range<0, kCopySlots>(l4, kStage);
+      in_flight = l4.count();
+    }
+    if (plan.total > 2) {
+      l4.advance();   // stays on stage 2: where the segment loop expects it
+      issue_range<0, kSplit>(l4, 2 * kStage);
+      in_flight += kSplit;
+    }
+  } else {
+    const GenericCopy g0(plan, 0, c);
+    issue_range<0, kCopySlots>(g0, lo, c.wave);
+    const GenericCopy g1(plan, 1, c);
+    issue_range<0, kCopySlots>(g1, lo, c.wave);
+    gc = GenericCopy(plan, 2, c);
+    issue_range<0, kSplit>(gc, lo, c.wave);
+    in_flight = g1.count() + (gc.b.seg < 0 ? 0 : kSplit);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
   v16f acc[4][TM];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
@@ -816,22 +863,9 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
     for (int b = 0; b < TM; ++b)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
+  __builtin_amdgcn_sched_barrier(0);
 
-  const LaneOffsets lo(plan, c);
-  const WeightPtrs wp(lds, c, TM);
-
-  // prologue: stages 0 and 1 and the first copies of stage 2 in flight; wait for stage 0 only
-  const int n4 = plan.st0, n6 = plan.st1, n8 = plan.st2;
-  GenericCopy gc;
-  {
-    const GenericCopy g0(plan, 0, c);
-    issue_range<0, kCopySlots>(g0, lo, c.wave);
-    const GenericCopy g1(plan, 1, c);
-    issue_range<0, kCopySlots>(g1, lo, c.wave);
-    gc = GenericCopy(plan, 2, c);
-    issue_range<0, kSplit>(gc, lo, c.wave);
-    wait_copies_but(g1.count() + (gc.b.seg < 0 ? 0 : kSplit));
-  }
+  wait_copies_but(in_flight);
   asm volatile("s_barrier" ::: "memory");
 
   static_assert(SEGS == 7 || (REGULAR && !REM && (SEGS == 1 || SEGS == 3 || SEGS == 5)), "plans with an empty segment");
@@ -847,11 +881,9 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
     wait_lds_reads();
     shift_scales(sc, sw, sx, c.lane, c.wm);
   }
-  LeanCopy<kFmtE2M1, WT> l4;
   LeanCopy<kFmtE3M2, WT> l6;
   LeanCopy<kFmtE4M3, WT> l8;
   LeanCopy<kFmtNone, WT> l0;
-  if constexpr (REGULAR) l4.init(plan, 2, lo, c);
   if constexpr (SEGS == 7) {
     run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
     run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR, NLAST>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
@@ -877,9 +909,10 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.
   // Each wave transposes its 128 tokens x 128 features through its own part of the (now idle)
   // LDS, so that a store instruction writes 4 rows x 256 contiguous bytes instead of 32 rows x 16.
+  // No barrier: the last stage reads no fragments after its barrier, before which every wave's copies had landed,
+  // and from here on a wave touches only its own part of the LDS.
   constexpr int kPitch = 256 + 16;   // bytes per token row in LDS
   static_assert(4 * 128 * kPitch <= kBuffers * kStage, "epilogue staging must fit the stage buffers");
-  __syncthreads();                   // every wave is done with the last stage's fragments
   uint8_t* stage = lds + c.wave * (32 * TM) * kPitch;
   {
     const int g = c.lane >> 5;

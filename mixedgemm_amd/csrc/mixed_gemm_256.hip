@@ -37,6 +37,7 @@ constexpr int kSOff = kXOff + 32 * kBlk;  // E4M3 worst case: two K halves x 16 
 constexpr int kStage = kSOff + 2048;      // 51968
 constexpr int kBuffers = 3;
 constexpr int kCopySlots = 13;            // 4 weight copies, up to 8 token copies, 1 scale copy per wave and stage
+constexpr int kStartSkew = 8000;          // see the kernel: largest start delay, in ticks of s_memtime (about 4 us)
 constexpr int kSplit = 5;                 // slots [0, kSplit) go out in the second half of a stage, the rest in the next first half
 
 typedef int v6i __attribute__((ext_vector_type(6)));
@@ -767,8 +768,18 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][TM], const uint8
 // NLAST: see run_segment (the launcher picks the instance from the plan).
 template <bool REGULAR, bool REM, bool WT, int SEGS = 7, int TM = 4, int NLAST = 0>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d) {
+mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d, int first_round,
+                      int skew) {
   extern __shared__ __align__(16) uint8_t lds[];
+  // Staggered start: with several tiles per CU, the first workgroup of each CU (the first `first_round` of the
+  // grid) starts up to `skew` clock ticks late, each by a different amount.  Every tile takes the same time, so
+  // without this all CUs load their first stages and store their result tiles in the same microseconds, tile after
+  // tile, and queue at the memory; the few microseconds lost once come back several times over.
+  if (skew > 0 && (int)blockIdx.x < first_round) {
+    const long long delay = (long long)skew * (((int)blockIdx.x >> 3) * 8 + ((int)blockIdx.x & 7)) / first_round;
+    const long long t0 = __builtin_amdgcn_s_memtime();
+    while ((long long)__builtin_amdgcn_s_memtime() - t0 < delay) __builtin_amdgcn_s_sleep(4);
+  }
   Plan plan;
   plan.a0 = uni(plan_arg.a0); plan.a1 = uni(plan_arg.a1); plan.a2 = uni(plan_arg.a2);
   plan.b0 = uni(plan_arg.b0); plan.b1 = uni(plan_arg.b1); plan.b2 = uni(plan_arg.b2);
@@ -986,7 +997,7 @@ static int tile_tokens(int m_store, int N) {
   return tiles <= 128 ? 128 : 256;
 }
 
-typedef void (*kernel_t)(Plan, int, int, int, int, uint16_t*);
+typedef void (*kernel_t)(Plan, int, int, int, int, uint16_t*, int, int);
 
 // The kernel for a plan: segs = which activation segments exist (bit 0 E2M1, 1 E3M2, 2 E4M3), nlast = stages of the
 // last one (3 = three or more).  Plans with an empty segment exist in the REGULAR, whole-stage form only.
@@ -1047,8 +1058,13 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   p.w_tiled = w_tiled ? 1 : 0;
   if (w_tiled && N % kT != 0) return hipErrorInvalidValue;
   const int tiles_n = (N + kT - 1) / kT, tiles_m = M / tokens;
-  hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store,
-                     a_rows, static_cast<uint16_t*>(d));
+  // more tiles than CUs: staggered start (see the kernel), up to kStartSkew ticks of the shader's clock counter
+  DeviceLimits lim;
+  if (hipError_t e = device_limits(&lim); e != hipSuccess) return e;
+  const int ntiles = tiles_n * tiles_m;
+  const int skew = ntiles > lim.cus ? kStartSkew : 0;
+  hipLaunchKernelGGL(kernel, dim3(ntiles), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,
+                     static_cast<uint16_t*>(d), lim.cus, skew);
   return hipGetLastError();
 }
 

@@ -554,7 +554,7 @@ struct Ring {
 // (FR == FMT) or `a_next`.  `xp` / `xpn`: token fragment addresses for FMT / FR.
 // LEAN: the late copy slots (of stage q+2, format CL) come from `lcl` when late_on, the early ones
 // (of stage q+3, format CE) from `lce` when early_on; MID says what happens to `lce` between the
-// halves: 1 = advance by one stage, 2 = set up for stage q+3 (first stage of its segment).
+// halves: 1 = advance by one stage, 2 = nothing (stage q+3 is the first of its segment, where lce stands).
 // !LEAN: both from the run-time plan `gc`.  next_on: there is a stage q+1.
 template <int FMT, int FR, bool LEAN, int CL, int CE, int MID, bool WT, int TM>
 __device__ __forceinline__ void stage_body(v16f (&acc)[4][TM], HalfFrags<FMT, TM>& a, HalfFrags<FR, TM>& a_next, Scales<TM>& sc,
@@ -580,8 +580,7 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][TM], HalfFrags<FMT, TM
   asm volatile("s_barrier" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
   if constexpr (LEAN) {
-    if constexpr (MID == 1) lce.advance();
-    else if constexpr (MID == 2) lce.init(plan, q + 3, lo, c);
+    if constexpr (MID == 1) lce.advance();   // MID == 2: lce was set up for its segment's first stage before the K loop
   } else {
     gc = GenericCopy(plan, q + 3, c);
   }
@@ -865,6 +864,14 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
     issue_range<0, kSplit>(gc, lo, c.wave);
     in_flight = g1.count() + (gc.b.seg < 0 ? 0 : kSplit);
   }
+  // the copy state of the later segments, while the first copies are in flight: set up between two halves of a
+  // stage it would hold up the MFMAs for several hundred cycles
+  LeanCopy<kFmtE3M2, WT> l6;
+  LeanCopy<kFmtE4M3, WT> l8;
+  if constexpr (REGULAR) {
+    if constexpr ((SEGS & 2) != 0) l6.init(plan, n4, lo, c);
+    if constexpr ((SEGS & 4) != 0) l8.init(plan, n4 + n6, lo, c);
+  }
   __builtin_amdgcn_sched_barrier(0);
 
   v16f acc[4][TM];
@@ -892,8 +899,6 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
     wait_lds_reads();
     shift_scales(sc, sw, sx, c.lane, c.wm);
   }
-  LeanCopy<kFmtE3M2, WT> l6;
-  LeanCopy<kFmtE4M3, WT> l8;
   LeanCopy<kFmtNone, WT> l0;
   if constexpr (SEGS == 7) {
     run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);

@@ -391,13 +391,24 @@ __device__ __forceinline__ void copy_region(const uint8_t* src, int bytes, unsig
 // to LDS as [step][piece]; piece_off is this lane's piece (lane % P) as a byte offset inside the atom (and, for
 // pieces of another group of 128 rows, that group's distance).  Units of 1 KB = 64 / P steps, unit u by wave u % 4;
 // steps past the last one copy it again (into the region's padding).
-__device__ __forceinline__ void copy_pieces(const uint8_t* src, int steps, int P, unsigned piece_off, unsigned dst,
+// P = 1 << plog pieces per step (a power of two: no divisions by a run-time value here)
+__device__ __forceinline__ void copy_pieces(const uint8_t* src, int steps, int plog, unsigned piece_off, unsigned dst,
                                             int wave, int lane) {
-  const int per_unit = 64 / P, units = (steps + per_unit - 1) / per_unit;
+  const int per_unit = 64 >> plog, units = (steps + per_unit - 1) >> (6 - plog);
   for (int u = wave; u < units; u += 4) {
-    const int q = min(u * per_unit + lane / P, steps - 1);
+    const int q = min(u * per_unit + (lane >> plog), steps - 1);
     dma16_at(src, (unsigned)q * 512u + piece_off, dst + (unsigned)u * 1024u);
   }
+}
+
+// All arguments into scalar registers in one batch of loads: fetched where they are first used they cost a round trip
+// to the argument buffer each time, before the first weight is requested.
+__device__ __forceinline__ void pin_args(DecodeSeg& s) {
+  asm volatile("" : "+s"(s.a), "+s"(s.b), "+s"(s.sfa), "+s"(s.sfb), "+s"(s.nblk), "+s"(s.steps));
+}
+__device__ __forceinline__ void pin_args(DecodeLds& l) {
+  asm volatile("" : "+s"(l.x0), "+s"(l.x1), "+s"(l.x2), "+s"(l.sfa0), "+s"(l.sfa1), "+s"(l.sfa2), "+s"(l.sfb0), "+s"(l.sfb1),
+               "+s"(l.sfb2), "+s"(l.partial), "+s"(l.total), "+s"(l.pa));
 }
 
 // 16 bytes global -> registers as an instruction the compiler does not count; use after s_waitcnt + tie()
@@ -414,7 +425,11 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
                          uint16_t* __restrict__ d) {
   constexpr int S = 4;        // K steps per round
   constexpr int PB = 4 * F;   // weight scale pieces per step
+  constexpr int PBLOG = F == 1 ? 2 : (F == 2 ? 3 : 4);
+  static_assert(F == 1 || F == 2 || F == 4, "pieces per step as a power of two");
   extern __shared__ __align__(16) uint8_t lds[];
+  pin_args(s4); pin_args(s6); pin_args(s8); pin_args(L);
+  asm volatile("" : "+s"(M), "+s"(N), "+s"(steps_per_wave), "+s"(d));
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, g = lane >> 4;
@@ -456,20 +471,6 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
     sfb_katoms_mul = group;
   }
 
-  // ---- what is not a weight code: requested first, into LDS
-  copy_region(s4.a, M * nblk4 * 16, lds0 + L.x0, wave, lane);
-  copy_region(s6.a, M * nblk6 * 24, lds0 + L.x1, wave, lane);
-  copy_region(s8.a, M * nblk8 * 32, lds0 + L.x2, wave, lane);
-  {
-    const unsigned pa_off = (unsigned)(lane % L.pa) * 16u;   // token scale pieces 0 ... pa - 1 of the first group of rows
-    if (s4.steps) copy_pieces(s4.sfa, s4.steps, L.pa, pa_off, lds0 + L.sfa0, wave, lane);
-    if (s6.steps) copy_pieces(s6.sfa, s6.steps, L.pa, pa_off, lds0 + L.sfa1, wave, lane);
-    if (s8.steps) copy_pieces(s8.sfa, s8.steps, L.pa, pa_off, lds0 + L.sfa2, wave, lane);
-    if (s4.steps) copy_pieces(s4.sfb, s4.steps, PB, sfb_piece_off + (unsigned)(sfb_katoms_mul * s4.steps) * 512u, lds0 + L.sfb0, wave, lane);
-    if (s6.steps) copy_pieces(s6.sfb, s6.steps, PB, sfb_piece_off + (unsigned)(sfb_katoms_mul * s6.steps) * 512u, lds0 + L.sfb1, wave, lane);
-    if (s8.steps) copy_pieces(s8.sfb, s8.steps, PB, sfb_piece_off + (unsigned)(sfb_katoms_mul * s8.steps) * 512u, lds0 + L.sfb2, wave, lane);
-  }
-
   // ---- weight codes: per lane 16 bytes per step and feature group (row n[f], block g of the step)
   int nc[F];
 #pragma unroll
@@ -498,10 +499,27 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
       }
     }
   };
-  if (rounds > 0) request_round(0, std::integral_constant<int, 0>{});
+  // ---- what is not a weight code, into LDS: requested first (measured: with the first round of weights ahead of
+  // them the kernel is slower, by 2 % on tile-major and 7 % on row-major weights)
+  copy_region(s4.a, M * nblk4 * 16, lds0 + L.x0, wave, lane);
+  copy_region(s6.a, M * nblk6 * 24, lds0 + L.x1, wave, lane);
+  copy_region(s8.a, M * nblk8 * 32, lds0 + L.x2, wave, lane);
+  {
+    const int palog = L.pa == 8 ? 3 : 4;
+    const unsigned pa_off = (unsigned)(lane & (L.pa - 1)) * 16u;   // token scale pieces 0 ... pa - 1 of the first group of rows
+    if (s4.steps) copy_pieces(s4.sfa, s4.steps, palog, pa_off, lds0 + L.sfa0, wave, lane);
+    if (s6.steps) copy_pieces(s6.sfa, s6.steps, palog, pa_off, lds0 + L.sfa1, wave, lane);
+    if (s8.steps) copy_pieces(s8.sfa, s8.steps, palog, pa_off, lds0 + L.sfa2, wave, lane);
+    if (s4.steps) copy_pieces(s4.sfb, s4.steps, PBLOG, sfb_piece_off + (unsigned)(sfb_katoms_mul * s4.steps) * 512u, lds0 + L.sfb0, wave, lane);
+    if (s6.steps) copy_pieces(s6.sfb, s6.steps, PBLOG, sfb_piece_off + (unsigned)(sfb_katoms_mul * s6.steps) * 512u, lds0 + L.sfb1, wave, lane);
+    if (s8.steps) copy_pieces(s8.sfb, s8.steps, PBLOG, sfb_piece_off + (unsigned)(sfb_katoms_mul * s8.steps) * 512u, lds0 + L.sfb2, wave, lane);
+  }
 
-  // ---- the copies are older than the weight requests: they are done when only those are in flight
-  if (rounds > 0) wait_vmcnt<S * F>();
+  if (rounds > 0) request_round(0, std::integral_constant<int, 0>{});
+  if (rounds > 1) request_round(1, std::integral_constant<int, 1>{});
+
+  // ---- the copies and the first round are older than the second round: done when only that is in flight
+  if (rounds > 1) wait_vmcnt<S * F>();
   else wait_vmcnt<0>();
   asm volatile("s_barrier" ::: "memory");
 
@@ -561,11 +579,22 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
 #pragma unroll
       for (int f = 0; f < F; ++f) tie(wq[B][k][f]);
   };
-  // Two rounds per iteration, both requested before the first is used; nothing is in flight across the loop edge
-  // (a register that an uncounted load is still to fill must not be moved by the compiler, which a value carried
-  // around a loop may be).  Round 0 is in flight already.
-  for (int r = 0; r < rounds; r += 2) {
-    if (r > 0) request_round(r, std::integral_constant<int, 0>{});
+  // Two rounds at a time, both requested before the first is used.  The first pair (requested above) is straight-line
+  // code, the loop requests its pairs itself: nothing is in flight across a loop edge (a register that an uncounted
+  // load is still to fill must not be moved by the compiler, which a value carried around a loop may be).
+  if (rounds > 0) {
+#pragma unroll
+    for (int k = 0; k < S; ++k)
+#pragma unroll
+      for (int f = 0; f < F; ++f) tie(wq[0][k][f]);
+    compute_round(0, std::integral_constant<int, 0>{});
+  }
+  if (rounds > 1) {
+    settle(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+    compute_round(1, std::integral_constant<int, 1>{});
+  }
+  for (int r = 2; r < rounds; r += 2) {
+    request_round(r, std::integral_constant<int, 0>{});
     if (r + 1 < rounds) {
       request_round(r + 1, std::integral_constant<int, 1>{});
       settle(std::integral_constant<int, 0>{}, std::integral_constant<int, S * F>{});
@@ -648,16 +677,21 @@ hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeS
   const int rows = M;
   // decode: the kernel that stages everything but the weight codes in LDS
   if (M <= 16 && ((d4.nblk | d6.nblk | d8.nblk) & 3) == 0) {
-    const int f = skinny_feature_groups(rows, N);
+    // feature groups of 16 per workgroup: 4 (tile-major weights; measured on N = 14336: 9.0 against 9.6 us) or 2 as
+    // long as that leaves most CUs a workgroup
+    int f = skinny_feature_groups(rows, N);
+    if (w_tiled && ceil_div(N, 64) >= 192) f = 4;
     DecodeLds L;
+    if (f == 4 && !decode_lds_plan(d4, d6, d8, M, f, &L)) f = 2;
     if (decode_lds_plan(d4, d6, d8, M, f, &L)) {
       const int spw = (d4.steps + d6.steps + d8.steps + 3) / 4;
       // row-major: per group of 128 rows 8 / F workgroups (the last group whole, rows past N clamped and not stored)
       const dim3 grid(w_tiled ? ceil_div(N, 16 * f) : ceil_div(N, 128) * (8 / f));
       typedef void (*kernel_t)(DecodeSeg, DecodeSeg, DecodeSeg, int, int, int, DecodeLds, uint16_t*);
-      const kernel_t kernels[2][2] = {{mixed_gemm_decode_kernel<1, false>, mixed_gemm_decode_kernel<2, false>},
-                                      {mixed_gemm_decode_kernel<1, true>, mixed_gemm_decode_kernel<2, true>}};
-      const kernel_t kernel = kernels[w_tiled ? 1 : 0][f - 1];
+      const kernel_t kernels[2][3] = {
+          {mixed_gemm_decode_kernel<1, false>, mixed_gemm_decode_kernel<2, false>, mixed_gemm_decode_kernel<4, false>},
+          {mixed_gemm_decode_kernel<1, true>, mixed_gemm_decode_kernel<2, true>, mixed_gemm_decode_kernel<4, true>}};
+      const kernel_t kernel = kernels[w_tiled ? 1 : 0][f == 4 ? 2 : f - 1];
       if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), 76 * 1024); e != hipSuccess) return e;
       hipLaunchKernelGGL(kernel, grid, dim3(256), (size_t)L.total, stream, d4, d6, d8, M, N, spw, L, d);
       return hipGetLastError();

@@ -192,6 +192,8 @@ DECODE_SHAPES = [
     (8, 14336, 2560, 1408, 128), (1, 4096, 2560, 1408, 128), (16, 512, 384, 256, 128), (7, 200, 128, 128, 128),
     (8, 8200, 256, 128, 0), (3, 1000, 2560, 1408, 128), (12, 136, 0, 384, 128), (8, 12288, 1280, 0, 256),
     (2, 9000, 4096, 2048, 512), (16, 8192, 128, 0, 0),
+    # wide tile-major layers: four feature groups per workgroup; 16 tokens, and K beyond the first two rounds
+    (16, 12288, 384, 256, 128), (5, 14336, 8960, 4928, 448),
 ]
 
 

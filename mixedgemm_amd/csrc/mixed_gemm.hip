@@ -415,6 +415,16 @@ __device__ __forceinline__ void pin_args(DecodeLds& l) {
 __device__ __forceinline__ void load16_uncounted(v4i& dst, const uint8_t* p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
 }
+// the same from a wave-uniform base (scalar registers), a 32-bit per-lane offset and an immediate: one instruction
+// per load and no 64-bit per-lane address arithmetic in front of it
+template <int OFF>
+__device__ __forceinline__ void load16_uncounted(v4i& dst, const uint8_t* sbase, unsigned voff) {
+  static_assert(OFF >= 0 && OFF < 4096, "immediate offset of a global load");
+  const uint64_t v = reinterpret_cast<uint64_t>(sbase);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  const uint64_t u = ((uint64_t)hi << 32) | lo;
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(voff), "s"(u), "n"(OFF) : "memory");
+}
 __device__ __forceinline__ void tie(v4i& r) { asm volatile("" : "+v"(r)); }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
@@ -476,6 +486,17 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
 #pragma unroll
   for (int f = 0; f < F; ++f) nc[f] = min(n[f], N - 1);   // clamped rows: every load is in bounds
   v4i wq[2][S][F];
+  // Per-lane byte offsets of the loads.  Tile-major: 16 KB per (256-feature tile, step), the workgroup's F blocks of
+  // 1 KB consecutive in it, lane quad i, piece g.  Row-major: row nc[f] of the segment, piece g of the step.
+  unsigned vrow4[F], vrow6[F], vrow8[F];
+  const unsigned vlane = (unsigned)(i * 64 + g * 16);
+#pragma unroll
+  for (int f = 0; f < F; ++f) {
+    vrow4[f] = (unsigned)nc[f] * (unsigned)nblk4 * 16u + (unsigned)g * 16u;
+    vrow6[f] = (unsigned)nc[f] * (unsigned)nblk6 * 16u + (unsigned)g * 16u;
+    vrow8[f] = (unsigned)nc[f] * (unsigned)nblk8 * 16u + (unsigned)g * 16u;
+  }
+  const int wtile = (blockIdx.x * F) >> 4, wj0 = (blockIdx.x * F) & 15;
   auto request_round = [&](int r, auto buf_c) {
     constexpr int B = decltype(buf_c)::value;
 #pragma unroll
@@ -484,18 +505,20 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
       const int seg = t < s4.steps ? 0 : (t < s4.steps + s6.steps ? 1 : 2);
       const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
       const uint8_t* pb = sel3p(seg, b4, b6, b8);
-      const int nblk = sel3(seg, nblk4, nblk6, nblk8);
-#pragma unroll
-      for (int f = 0; f < F; ++f) {
-        const uint8_t* p;
-        if constexpr (WT) {
-          // 16 KB per (256-feature tile, step), the block's 1 KB in it, lane quad i, piece g
-          const int bx = blockIdx.x * F + f;
-          p = pb + ((((size_t)(bx >> 4) * (nblk >> 2) + q) * 16 + (bx & 15)) * 1024 + i * 64 + g * 16);
-        } else {
-          p = pb + (size_t)nc[f] * nblk * 16 + q * 64 + g * 16;
+      if constexpr (WT) {
+        const int nst = sel3(seg, nblk4, nblk6, nblk8) >> 2;
+        const uint8_t* sb = pb + (((size_t)wtile * nst + q) * 16 + wj0) * 1024;
+        if constexpr (F >= 1) load16_uncounted<0>(wq[B][k][0], sb, vlane);
+        if constexpr (F >= 2) load16_uncounted<1024>(wq[B][k][F >= 2 ? 1 : 0], sb, vlane);
+        if constexpr (F >= 4) {
+          load16_uncounted<2048>(wq[B][k][F >= 4 ? 2 : 0], sb, vlane);
+          load16_uncounted<3072>(wq[B][k][F >= 4 ? 3 : 0], sb, vlane);
         }
-        load16_uncounted(wq[B][k][f], p);
+      } else {
+        const uint8_t* sb = pb + (size_t)q * 64;
+#pragma unroll
+        for (int f = 0; f < F; ++f)
+          load16_uncounted<0>(wq[B][k][f], sb, (unsigned)sel3(seg, (int)vrow4[f], (int)vrow6[f], (int)vrow8[f]));
       }
     }
   };
@@ -676,7 +699,9 @@ hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeS
                          bool w_tiled, uint16_t* d, hipStream_t stream) {
   const int rows = M;
   // decode: the kernel that stages everything but the weight codes in LDS
-  if (M <= 16 && ((d4.nblk | d6.nblk | d8.nblk) & 3) == 0) {
+  // (a segment's weight codes below 4 GB: the kernel addresses them with 32-bit per-lane offsets)
+  const size_t widest = (size_t)(d4.nblk > d6.nblk ? (d4.nblk > d8.nblk ? d4.nblk : d8.nblk) : (d6.nblk > d8.nblk ? d6.nblk : d8.nblk));
+  if (M <= 16 && ((d4.nblk | d6.nblk | d8.nblk) & 3) == 0 && (size_t)N * widest * 16 < ((size_t)1 << 32)) {
     // feature groups of 16 per workgroup: 4 (tile-major weights; measured on N = 14336: 9.0 against 9.6 us) or 2 as
     // long as that leaves most CUs a workgroup
     int f = skinny_feature_groups(rows, N);

@@ -36,13 +36,13 @@ P46, P8 = 10100.0, 5000.0
 # of the kernel source it was taken with; when the source has changed since, the JSON carries null and says so.
 PROFILE = "profiles/hbm_traffic_fetch_write_size.txt"
 MEASURED_TRAFFIC = {
-    "gemm_c3": {"bytes": int((136016.6 * 1.99981 + 115681.4 * 1.0) * 1024),      # 397 MB against 159 MB algorithmic: operands re-read 6.8x past L2
-                "source": "mixedgemm_amd/csrc/mixed_gemm_256.hip", "sha": "a805d6deffd5d4f2"},
-    "quant_c1": {"bytes": int((16465.5 * 1.99981 + 10528.6 * 1.0) * 1024),       # 44.5 MB against 44.2 MB algorithmic
+    "gemm_c3": {"bytes": int((110287.6 * 1.99981 + 114755.8 * 1.0) * 1024),      # 343 MB against 159 MB algorithmic: operands re-read 5.5x past L2
+                "source": "mixedgemm_amd/csrc/mixed_gemm_256.hip", "sha": "07e2a66bf01c9480"},
+    "quant_c1": {"bytes": int((16465.5 * 1.99981 + 10531.8 * 1.0) * 1024),       # 44.5 MB against 44.2 MB algorithmic
                  "source": "mixedgemm_amd/csrc/reorder_quant.hip", "sha": "46e30380386eea83"},
-    "decode_c2": {"bytes": int((15443.0 * 1.99981 + 448.0 * 1.0) * 1024),        # 32.1 MB against 31.4 MB algorithmic
-                  "source": "mixedgemm_amd/csrc/mixed_gemm.hip", "sha": "2e42fb6d18361bac"},
-    "calibrate_c1": {"bytes": int(((16411.0 + 1043.4 + 81.5) * 1.99981 + (2048.0 + 16.0 + 56.3) * 1.0) * 1024),   # three kernels
+    "decode_c2": {"bytes": int((16318.0 * 1.99981 + 896.0 * 1.0) * 1024),        # 34.3 MB against 31.4 MB algorithmic (tile-major weights)
+                  "source": "mixedgemm_amd/csrc/mixed_gemm.hip", "sha": "8241005004ff8775"},
+    "calibrate_c1": {"bytes": int(((16411.0 + 1045.0 + 81.5) * 1.99981 + (2048.0 + 16.0 + 56.2) * 1.0) * 1024),   # three kernels
                      "source": "mixedgemm_amd/csrc/calibrate.hip", "sha": "84a260f8dfd73ec0"},
 }
 
@@ -389,28 +389,36 @@ def main():
         idx2 = H.absmax_sort_index(x2).to(dev)
         aq2 = abi.reorder_quantize_x(x2.to(dev), idx2, kn2, ks2, ko2)
         nsets2 = 10                                  # 10 x 31 MB of weights > 256 MB
-        wq = [abi.reorder_quantize_w(H.make_weights(n2, k2, 3000 + i).to(dev), idx2, kn2, ks2, ko2) for i in range(nsets2)]
+        wq_rm = [abi.reorder_quantize_w(H.make_weights(n2, k2, 3000 + i).to(dev), idx2, kn2, ks2, ko2) for i in range(nsets2)]
+        # tile-major codes: the layout the packed weights of a layer are stored in (as in the headline's step)
+        wq = [abi.tile_weights(*b[:3]) + b[3:] for b in wq_rm]
         d2 = torch.empty((m2, n2), dtype=torch.bfloat16, device=dev)
-        for i in range(args.warmup + nsets2):
-            b = wq[i % nsets2]
-            abi.matmul(aq2[0], b[0], aq2[1], b[1], aq2[2], b[2], aq2[3], b[3], aq2[4], b[4], aq2[5], b[5], out=d2)
-        torch.cuda.synchronize()
+
         def decode(i):
             b = wq[i % nsets2]
+            abi.matmul(aq2[0], b[0], aq2[1], b[1], aq2[2], b[2], aq2[3], b[3], aq2[4], b[4], aq2[5], b[5], out=d2, w_tiled=True)
+
+        def decode_rm(i):
+            b = wq_rm[i % nsets2]
             abi.matmul(aq2[0], b[0], aq2[1], b[1], aq2[2], b[2], aq2[3], b[3], aq2[4], b[4], aq2[5], b[5], out=d2)
 
+        for i in range(args.warmup + nsets2):
+            decode(i)
+            decode_rm(i)
+        torch.cuda.synchronize()
+        g_rm_ms = graph_ms(decode_rm, iters)
         g_ms = graph_ms(decode, iters)
         gb = gemm_bytes(m2, n2, kn2, ks2, ko2)
         g_gbs = gb / (g_ms * 1e-3) / 1e9
         extra["decode_gemm_c2"] = {
-            "workload": "c2 mixed GEMM M=8 K=4096 (2560/1408/128) N=14336, 10 rotating weight sets",
-            "value": round(g_gbs, 1), "unit": "GB/s", "avg_kernel_ms": round(g_ms, 5),
+            "workload": "c2 mixed GEMM M=8 K=4096 (2560/1408/128) N=14336, tile-major weight codes, 10 rotating weight sets",
+            "value": round(g_gbs, 1), "unit": "GB/s", "avg_kernel_ms": round(g_ms, 5), "row_major_weights_ms": round(g_rm_ms, 5),
             "tflops": round(2.0 * m2 * n2 * k2 / (g_ms * 1e-3) / 1e12, 3),
             "roofline": {"bound": "hbm", "achieved": round(g_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(g_gbs / HBM_PEAK_GBS, 4), "traffic": traffic("decode_c2")[0], "traffic_source": traffic("decode_c2")[1],
                          "algorithmic_bytes": gb},
         }
-        del wq
+        del wq, wq_rm
 
         # ------------------------------------------------------------ the other layer shapes of the reference's K list
         # fused step (activation reorder-quantize + mixed GEMM) per shape; weights quantized outside the timing

@@ -11,7 +11,7 @@ namespace mg {
 template <bool IS_W>
 hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int K, int KN, int KS, int KO, uint8_t* qn,
                                 uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, const void* gamma,
-                                float eps, hipStream_t stream);
+                                float eps, bool keep_codes, hipStream_t stream);
 hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                              const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                              const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo, int M,
@@ -39,14 +39,14 @@ int check_split(int rows, int KN, int KS, int KO) {
 template <bool IS_W>
 int reorder_quantize(const void* x, const int16_t* idx, int rows, int K, int KN, int KS, int KO, uint8_t* qn,
                      uint8_t* qs, uint8_t* qo, uint8_t* sfn, uint8_t* sfs, uint8_t* sfo, void* stream,
-                     const void* gamma = nullptr, float eps = 0.0f) {
+                     const void* gamma = nullptr, float eps = 0.0f, bool keep_codes = false) {
   if (int s = check_split(rows, KN, KS, KO)) return s;
   if (K != KN + KS + KO) return MG_ERR_BAD_SHAPE;
   if (rows == 0 || K == 0) return MG_OK;
   if (!ptr_ok(x, true) || !ptr_ok(idx, true)) return MG_ERR_BAD_POINTER;
   if (!ptr_ok(qn, KN > 0) || !ptr_ok(qs, KS > 0) || !ptr_ok(qo, KO > 0)) return MG_ERR_BAD_POINTER;
   if ((KN > 0 && !sfn) || (KS > 0 && !sfs) || (KO > 0 && !sfo)) return MG_ERR_BAD_POINTER;
-  return (int)mg::launch_reorder_quant<IS_W>(x, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, gamma, eps,
+  return (int)mg::launch_reorder_quant<IS_W>(x, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, gamma, eps, keep_codes,
                                              static_cast<hipStream_t>(stream));
 }
 
@@ -179,7 +179,9 @@ int mg_fused_norm_linear(const void* x_bf16, const void* gamma_bf16, float eps, 
   uint8_t* sfn = p; p += align256(mg_sf_bytes(R, KN, MG_OPERAND_A));
   uint8_t* sfs = p; p += align256(mg_sf_bytes(R, KS, MG_OPERAND_A));
   uint8_t* sfo = p;
-  if (int s = reorder_quantize<false>(x_bf16, idx, M, KN + KS + KO, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream, gamma_bf16, eps))
+  // the GEMM reads the codes next: ordinary stores, so that they are in the L2 when it starts
+  if (int s = reorder_quantize<false>(x_bf16, idx, M, KN + KS + KO, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream, gamma_bf16, eps,
+                                      /*keep_codes=*/true))
     return s;
   return mg_mixed_gemm_ex(qn, bn, qs, bs, qo, bo, sfn, sfbn, sfs, sfbs, sfo, sfbo, M, R, N, KN, KS, KO, flags, d_bf16, stream);
 }

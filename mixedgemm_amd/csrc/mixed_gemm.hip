@@ -690,22 +690,24 @@ static bool decode_lds_plan(const DecodeSeg& d4, const DecodeSeg& d6, const Deco
 }
 
 // Feature groups of 16 per workgroup of the skinny kernel.
-static int skinny_feature_groups(int rows, int N) {
+static int skinny_feature_groups(int rows, int N, int cus) {
   const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
-  return ceil_div(N, 32) * ceil_div(rows, 16 * g) >= 256 ? 2 : 1;
+  return ceil_div(N, 32) * ceil_div(rows, 16 * g) >= cus ? 2 : 1;
 }
 
 hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int N,
                          bool w_tiled, uint16_t* d, hipStream_t stream) {
   const int rows = M;
+  DeviceLimits lim;
+  if (hipError_t e = device_limits(&lim); e != hipSuccess) return e;
   // decode: the kernel that stages everything but the weight codes in LDS
   // (a segment's weight codes below 4 GB: the kernel addresses them with 32-bit per-lane offsets)
   const size_t widest = (size_t)(d4.nblk > d6.nblk ? (d4.nblk > d8.nblk ? d4.nblk : d8.nblk) : (d6.nblk > d8.nblk ? d6.nblk : d8.nblk));
   if (M <= 16 && ((d4.nblk | d6.nblk | d8.nblk) & 3) == 0 && (size_t)N * widest * 16 < ((size_t)1 << 32)) {
     // feature groups of 16 per workgroup: 4 (tile-major weights; measured on N = 14336: 9.0 against 9.6 us) or 2 as
     // long as that leaves most CUs a workgroup
-    int f = skinny_feature_groups(rows, N);
-    if (w_tiled && ceil_div(N, 64) >= 192) f = 4;
+    int f = skinny_feature_groups(rows, N, lim.cus);
+    if (w_tiled && ceil_div(N, 64) >= lim.cus * 3 / 4) f = 4;
     DecodeLds L;
     if (f == 4 && !decode_lds_plan(d4, d6, d8, M, f, &L)) f = 2;
     if (decode_lds_plan(d4, d6, d8, M, f, &L)) {
@@ -727,7 +729,7 @@ hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeS
   // two feature groups per workgroup for 17-64 tokens: each activation fragment then serves 32 features
   // two feature groups per workgroup (an activation fragment then serves 32 features) as long as that
   // leaves a workgroup for every CU; measured on N = 2048 ... 14336
-  const int f = skinny_feature_groups(rows, N);
+  const int f = skinny_feature_groups(rows, N, lim.cus);
   const dim3 grid(ceil_div(N, 16 * f), ceil_div(rows, 16 * g));
   const int wt = w_tiled ? 1 : 0;
   switch (g) {
@@ -1053,7 +1055,7 @@ static double pipelined_us(int m_pad, int N, int stages) {
   return (double)((tiles + 255) / 256) * (stages * (tiles <= 128 ? 0.7 : 1.05) + 8.0);
 }
 static double skinny_us(int rows, int N, int steps) {
-  const double per_unit = skinny_feature_groups(rows, N) == 2 ? 0.19e-3 : 0.25e-3;
+  const double per_unit = skinny_feature_groups(rows, N, 256) == 2 ? 0.19e-3 : 0.25e-3;   // (the figures are MI355X's: 256 CUs)
   return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * per_unit;
 }
 

@@ -997,9 +997,9 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
 // at least half of the CUs without one.  A half tile takes about 0.8 of a whole tile's time (the copies of a stage
 // bound it, not its MFMAs), so halves pay only where they put idle CUs to work: measured, M = 2048 N = 4096
 // K = 14336 (128 whole tiles) 99 -> 84 us, M = 1024 N = 4096 K = 4096 (64) 28 -> 22 us, but 896 whole tiles 145 -> 170 us.
-static int tile_tokens(int m_store, int N) {
+static int tile_tokens(int m_store, int N, int cus) {
   const long long tiles = (long long)((m_store + kT - 1) / kT) * ((N + kT - 1) / kT);
-  return tiles <= 128 ? 128 : 256;
+  return tiles <= cus / 2 ? 128 : 256;
 }
 
 typedef void (*kernel_t)(Plan, int, int, int, int, uint16_t*, int, int);
@@ -1033,7 +1033,9 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   // m_store tokens are computed in whole tiles of 256 or 128 token rows; rows past m_store are computed but not
   // stored; the activation buffers are read up to row a_rows - 1 only
   if (m_store <= 0 || a_rows < m_store) return hipErrorInvalidValue;
-  const int tokens = tile_tokens(m_store, N);
+  DeviceLimits lim;
+  if (hipError_t e = device_limits(&lim); e != hipSuccess) return e;
+  const int tokens = tile_tokens(m_store, N, lim.cus);
   const int M = (m_store + tokens - 1) / tokens * tokens;
   // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
   const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
@@ -1064,8 +1066,6 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   if (w_tiled && N % kT != 0) return hipErrorInvalidValue;
   const int tiles_n = (N + kT - 1) / kT, tiles_m = M / tokens;
   // more tiles than CUs: staggered start (see the kernel), up to kStartSkew ticks of the shader's clock counter
-  DeviceLimits lim;
-  if (hipError_t e = device_limits(&lim); e != hipSuccess) return e;
   const int ntiles = tiles_n * tiles_m;
   const int skew = ntiles > lim.cus ? kStartSkew : 0;
   hipLaunchKernelGGL(kernel, dim3(ntiles), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,

@@ -128,223 +128,8 @@ __device__ __forceinline__ void quantize_store(const float (&f)[32], int fmt, ui
   }
 }
 
-// A workgroup handles groups of R consecutive rows, group blockIdx.x first and then every
-// gridDim.x-th one; blockDim.x >= K/32 (at most MAXT).  The global loads of the next group are
-// issued before the current group is gathered and quantized, and the LDS tile is double buffered
-// (buf_stride bytes apart; 0 when every workgroup has a single group), so loads, arithmetic and
-// stores of different groups overlap inside the workgroup and one barrier per group suffices.
-//
-// NORM: an RMSNorm (weight gamma, bf16 in and out, the arithmetic of the usual fp32 implementation)
-// is applied to each row before the gather:
-//   var = fl32( (sum over the row of x^2, accumulated in fp64) / K )
-//   r   = fl32( 1 / sqrt( fl32(var + eps) ) )      (division and square root in fp64)
-//   y   = bf16( gamma * bf16( x * r ) )            (both products in fp32)
-// The fp64 sum makes the result independent of the order in which the lanes add their parts
-// (up to the last bit of a double, which the rounding to fp32 all but never sees).
-template <int R, bool IS_W, int MAXT, bool NORM>
-__global__ void __launch_bounds__(MAXT)
-reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__ idx, int rows, int K, int KN, int KS,
-                     int KO, uint8_t* __restrict__ qn, uint8_t* __restrict__ qs, uint8_t* __restrict__ qo,
-                     uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo, int buf_stride,
-                     const uint16_t* __restrict__ gamma, float eps) {
-  extern __shared__ __align__(16) uint8_t lds_all[];
-  __shared__ double row_sums[R][MAXT / 64];
-  const int tid = threadIdx.x;
-  const int nthr = blockDim.x;
-  const int ngroups = (rows + R - 1) / R;
-
-  // ---- the lane's 32 reorder indices (the same for every row): requested first, needed only
-  //      after the first barrier
-  const int b = tid;
-  const bool has_block = b < (K >> 5);
-  v4u iv[4];
-  {
-    const v4u* ip = reinterpret_cast<const v4u*>(idx + (size_t)(has_block ? b : 0) * 32);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) iv[q] = ip[q];
-  }
-
-  // per-lane block constants
-  const int nbn = KN >> 5, nbs = KS >> 5;
-  const int seg = b < nbn ? 0 : (b < nbn + nbs ? 1 : 2);
-  const int j = seg == 0 ? b : (seg == 1 ? b - nbn : b - nbn - nbs);
-  const int kseg = seg == 0 ? KN : (seg == 1 ? KS : KO);
-  const int katoms = (kseg + 127) >> 7;
-  const int fmt = IS_W ? kFmtE2M1 : (seg == 0 ? kFmtE2M1 : (seg == 1 ? kFmtE3M2 : kFmtE4M3));
-  const int blk_bytes = fmt == kFmtE2M1 ? 16 : (fmt == kFmtE3M2 ? 24 : 32);
-  const size_t pitch = (size_t)(kseg >> 5) * blk_bytes;
-  uint8_t* qbase = (seg == 0 ? qn : (seg == 1 ? qs : qo)) + j * blk_bytes;
-  uint8_t* sfbase = seg == 0 ? sfn : (seg == 1 ? sfs : sfo);
-
-  // ---- stage R rows: all 16-byte loads issued up front (row and chunk clamped instead of
-  //      branched, so nothing waits), R x 8 transpose in registers, 16-byte LDS stores.
-  //      Channel c of row r lands at lds[(c*R + r)*2].
-  const int nchunks = K >> 3;
-  v4u a[4][R];
-  auto issue_loads = [&](int group) {
-    const int row0 = group * R;
-#pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int c = min(tid + it * nthr, nchunks - 1);
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int row = min(row0 + r, rows - 1);
-        a[it][r] = *reinterpret_cast<const v4u*>(x + (size_t)row * K + (size_t)c * 8);
-      }
-    }
-  };
-
-  int group = blockIdx.x;
-  if (group >= ngroups) return;
-  issue_loads(group);
-  v4u gv[4];   // the RMSNorm weights of this lane's chunks (the same for every row)
-  if constexpr (NORM) {
-#pragma unroll
-    for (int it = 0; it < 4; ++it)
-      gv[it] = *reinterpret_cast<const v4u*>(gamma + (size_t)min(tid + it * nthr, nchunks - 1) * 8);
-  }
-  // Byte offsets of the lane's 32 gathered channels inside a tile (the same for every row).  An entry outside
-  // [0, K) is read as channel K - 1, so that the gather stays inside the tile whatever the index holds.
-  unsigned ga[32];
-#pragma unroll
-  for (int q = 0; q < 4; ++q)
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      ga[q * 8 + e] = min((e & 1) ? (iv[q][e >> 1] >> 16) : (iv[q][e >> 1] & 0xffffu), (unsigned)(K - 1)) * (2 * R);
-
-  // The loop body exists once per LDS buffer, so that the buffer's offset is a compile-time
-  // constant wherever the buffers are a fixed distance apart (kFixed) and folds into the LDS
-  // instructions' immediate offsets: the gather is then one instruction per channel.
-  constexpr bool kFixed = MAXT == 256;
-  constexpr int kBuf1 = MAXT * 64 * R;   // largest tile of this instantiation
-  auto body = [&](auto parity_c) {
-    constexpr int parity = decltype(parity_c)::value;
-    uint8_t* lds = lds_all + (kFixed ? parity * kBuf1 : parity * buf_stride);
-    const int row0 = group * R;
-    if constexpr (NORM) {
-      double ss[R];
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        ss[r] = 0.0;
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-          if (tid + it * nthr < nchunks) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const unsigned d = a[it][r][e];
-              const double lo = (double)__uint_as_float(d << 16), hi = (double)__uint_as_float(d & 0xffff0000u);
-              ss[r] = __builtin_fma(lo, lo, ss[r]);
-              ss[r] = __builtin_fma(hi, hi, ss[r]);
-            }
-          }
-        }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) ss[r] += __shfl_xor(ss[r], off, 64);
-        if ((tid & 63) == 0) row_sums[r][tid >> 6] = ss[r];
-      }
-      __syncthreads();
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        double tot = 0.0;
-        for (int w = 0; w < (nthr >> 6); ++w) tot += row_sums[r][w];
-        const float var = (float)(tot / (double)K);
-        const float rn = (float)(1.0 / __builtin_sqrt((double)(var + eps)));
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const unsigned d = a[it][r][e], g = gv[it][e];
-            const float h0 = (float)(__bf16)(__uint_as_float(d << 16) * rn);
-            const float h1 = (float)(__bf16)(__uint_as_float(d & 0xffff0000u) * rn);
-            const v2bf y = {(__bf16)(__uint_as_float(g << 16) * h0), (__bf16)(__uint_as_float(g & 0xffff0000u) * h1)};
-            a[it][r][e] = __builtin_bit_cast(unsigned, y);
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int c = tid + it * nthr;
-      if (c < nchunks) {
-        v4u* dst = reinterpret_cast<v4u*>(lds + (size_t)c * 16 * R);
-        if constexpr (R == 1) {
-          dst[0] = a[it][0];
-        } else if constexpr (R == 2) {
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            v4u o;
-            o[0] = perm(a[it][1][2 * h], a[it][0][2 * h], 0x05040100u);
-            o[1] = perm(a[it][1][2 * h], a[it][0][2 * h], 0x07060302u);
-            o[2] = perm(a[it][1][2 * h + 1], a[it][0][2 * h + 1], 0x05040100u);
-            o[3] = perm(a[it][1][2 * h + 1], a[it][0][2 * h + 1], 0x07060302u);
-            dst[h] = o;
-          }
-        } else {
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj) {
-            v4u o;
-            o[0] = perm(a[it][1][jj], a[it][0][jj], 0x05040100u);
-            o[1] = perm(a[it][3][jj], a[it][2][jj], 0x05040100u);
-            o[2] = perm(a[it][1][jj], a[it][0][jj], 0x07060302u);
-            o[3] = perm(a[it][3][jj], a[it][2][jj], 0x07060302u);
-            dst[jj] = o;
-          }
-        }
-      }
-    }
-    __syncthreads();
-    // the registers are free again: request the next group's rows while this one is processed
-    if (group + (int)gridDim.x < ngroups) issue_loads(group + gridDim.x);
-
-    // ---- one lane per 32-element block
-    if (has_block) {
-      unsigned g[32][(R + 1) / 2];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int p = q * 8 + e;
-          if constexpr (R == 4) {
-            const v2u d = *reinterpret_cast<const v2u*>(lds + ga[p]);
-            g[p][0] = d[0];
-            g[p][1] = d[1];
-          } else if constexpr (R == 2) {
-            g[p][0] = *reinterpret_cast<const unsigned*>(lds + ga[p]);
-          } else {
-            g[p][0] = *reinterpret_cast<const uint16_t*>(lds + ga[p]);
-          }
-        }
-      }
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int row = row0 + r;
-        if (row >= rows) break;
-        float f[32];
-#pragma unroll
-        for (int p = 0; p < 32; ++p) {
-          const unsigned d = g[p][r >> 1];
-          f[p] = __uint_as_float((r & 1) ? (d & 0xffff0000u) : (d << 16));
-        }
-        // per-lane format, code row pitch and byte offset of the block inside its row
-        quantize_store(f, fmt, qbase + (size_t)row * pitch, sfbase + sf_offset(row, j, katoms));
-      }
-    }
-    // with one buffer (buf_stride == 0) there is exactly one group per workgroup; with two, the
-    // barrier of the next iteration separates this gather from the stores two iterations on
-  };
-  while (true) {
-    body(std::integral_constant<int, 0>{});
-    group += gridDim.x;
-    if (group >= ngroups) break;
-    body(std::integral_constant<int, 1>{});
-    group += gridDim.x;
-    if (group >= ngroups) break;
-  }
-}
-
-
 // ---------------------------------------------------------------------------------------------
-// The kernel without RMSNorm (activations and weights): rows go global -> LDS directly.
+// The kernel (activations and weights): rows go global -> LDS directly.
 //
 // A workgroup owns rows first, first + gridDim.x, ... and a ring of NS row slots in LDS (row-major, as in
 // memory).  The rows of the first NS iterations are requested before anything else happens
@@ -363,6 +148,31 @@ reorder_quant_kernel(const uint16_t* __restrict__ x, const int16_t* __restrict__
 // T > 0: blockDim.x == T and the slot offsets are immediates of the LDS reads; T == 0: any blockDim.x, the
 // slot offset is added to the addresses per row.
 // ---------------------------------------------------------------------------------------------
+// Sum of a double over the 64 lanes of a wave, the same value in every lane: four data-parallel-primitive steps inside
+// the rows of 16 lanes (two register moves and an add each, no trip through the LDS crossbar), then the four row sums
+// through scalar registers.
+template <int CTRL>
+__device__ __forceinline__ double dpp_add(double v) {
+  const uint64_t b = __builtin_bit_cast(uint64_t, v);
+  const int lo = __builtin_amdgcn_mov_dpp((int)(uint32_t)b, CTRL, 0xF, 0xF, true);
+  const int hi = __builtin_amdgcn_mov_dpp((int)(uint32_t)(b >> 32), CTRL, 0xF, 0xF, true);
+  return v + __builtin_bit_cast(double, ((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo);
+}
+__device__ __forceinline__ double wave_sum(double v) {
+  v = dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  v = dpp_add<0x141>(v);   // row_half_mirror: the other quad of the 8
+  v = dpp_add<0x140>(v);   // row_mirror: the other 8 of the 16
+  const uint64_t b = __builtin_bit_cast(uint64_t, v);
+  double rows[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)b, 16 * r), hi = __builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), 16 * r);
+    rows[r] = __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+  }
+  return (rows[0] + rows[1]) + (rows[2] + rows[3]);
+}
+
 __device__ __forceinline__ void dma16(const uint8_t* base, unsigned voff, unsigned lds_off) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                : : "v"(voff), "s"(base), "s"(lds_off) : "memory", "m0");
@@ -472,12 +282,14 @@ struct RowSchedule {
   int width[3];   // then: the first width[j] workgroups take one (0: nobody)
 };
 
-template <int EPL, int T, int NS, bool IS_W, int MAXT, bool KEEP = false>
+template <int EPL, int T, int NS, bool IS_W, int MAXT, bool KEEP = false, bool NORM = false>
 __global__ void __launch_bounds__(MAXT)
 reorder_quant_dma_kernel(const uint8_t* __restrict__ x, const int16_t* __restrict__ idx, int rows, int K, int KN, int KS,
                          int KO, uint8_t* __restrict__ qn, uint8_t* __restrict__ qs, uint8_t* __restrict__ qo,
-                         uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo, RowSchedule sched) {
+                         uint8_t* __restrict__ sfn, uint8_t* __restrict__ sfs, uint8_t* __restrict__ sfo, RowSchedule sched,
+                         const uint16_t* __restrict__ gamma, float eps) {
   extern __shared__ __align__(16) uint8_t lds[];
+  __shared__ double row_sums[NORM ? 2 : 1][NORM ? MAXT / 64 : 1];   // RMSNorm: the waves' sums of squares, by row parity
   static_assert(EPL == 32 || EPL == 16, "one or two lanes per block");
   constexpr int kPieces = EPL / 8;   // 16-byte pieces of a row (and of the index) per lane
   constexpr int kParts = EPL / 16;   // gathers of 16 per lane and row
@@ -546,6 +358,14 @@ reorder_quant_dma_kernel(const uint8_t* __restrict__ x, const int16_t* __restric
 #pragma unroll
   for (int s = 0; s < NS; ++s)
     if (s < count) request(x + (size_t)row_of(s) * row_bytes, s * stride);
+  // RMSNorm: the weights of this lane's pieces of a row (the same for every row); ordinary loads, which the compiler
+  // waits for itself where they are first used (with vmcnt(0): once, in the first row)
+  v4u gv[kPieces];
+  if constexpr (NORM) {
+#pragma unroll
+    for (int it = 0; it < kPieces; ++it)
+      gv[it] = *reinterpret_cast<const v4u*>(gamma + (size_t)min(it * nthr + tid, nchunks - 1) * 8);
+  }
 
   const int nbn = KN >> 5, nbs = KS >> 5;
   const int seg = b < nbn ? 0 : (b < nbn + nbs ? 1 : 2);
@@ -591,10 +411,59 @@ reorder_quant_dma_kernel(const uint8_t* __restrict__ x, const int16_t* __restric
     // in order): the requests of the rows after it -- NS - 1 of them at the start, NS - 2 once refills follow the
     // iterations -- and the stores of the iterations since, at most NS - 1 of them.
     wait_vm(kPieces * min(i == 0 ? NS - 1 : NS - 2, count - 1 - i) + row_stores * min(i, NS - 1));
-    asm volatile("s_barrier" ::: "memory");
-    // every wave is past its gather of row i - 1: refill that row's slot
-    if (i >= 1 && i - 1 + NS < count)
-      request(x + (size_t)row_of(i + NS - 1) * row_bytes, ((S + NS - 1) % NS) * stride);
+    if constexpr (NORM) {
+      // RMSNorm of the row, in place, before anyone gathers from it (the arithmetic of the usual fp32 implementation):
+      //   var = fl32( (sum over the row of x^2, accumulated in fp64) / K )
+      //   r   = fl32( 1 / sqrt( fl32(var + eps) ) )      (division and square root in fp64)
+      //   y   = bf16( gamma * bf16( x * r ) )            (both products in fp32)
+      // The fp64 sum makes the result independent of the order in which the lanes add their parts (up to the last
+      // bit of a double, which the rounding to fp32 all but never sees).  A lane works on the pieces it copied.
+      uint8_t* slot = lds + S * stride;
+      v4u a[kPieces];
+      double ss = 0.0;
+#pragma unroll
+      for (int it = 0; it < kPieces; ++it) {
+        a[it] = *reinterpret_cast<const v4u*>(slot + (size_t)(it * nthr + tid) * 16);
+        if (it * nthr + tid < nchunks) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const unsigned d = a[it][e];
+            const double lo = (double)__uint_as_float(d << 16), hi = (double)__uint_as_float(d & 0xffff0000u);
+            ss = __builtin_fma(lo, lo, ss);
+            ss = __builtin_fma(hi, hi, ss);
+          }
+        }
+      }
+      ss = wave_sum(ss);
+      if ((tid & 63) == 0) row_sums[i & 1][tid >> 6] = ss;
+      __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the sum is in the LDS (a raw barrier implies no wait of the compiler's)
+      asm volatile("s_barrier" ::: "memory");   // also: every wave's copies of row i have landed, every wave is past its gather of row i - 1
+      if (i >= 1 && i - 1 + NS < count)
+        request(x + (size_t)row_of(i + NS - 1) * row_bytes, ((S + NS - 1) % NS) * stride);
+      double tot = 0.0;
+      for (int w = 0; w < (nthr >> 6); ++w) tot += row_sums[i & 1][w];
+      const float var = (float)(tot / (double)K);
+      const float rn = (float)(1.0 / __builtin_sqrt((double)(var + eps)));
+#pragma unroll
+      for (int it = 0; it < kPieces; ++it) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const unsigned d = a[it][e], g = gv[it][e];
+          const float h0 = (float)(__bf16)(__uint_as_float(d << 16) * rn);
+          const float h1 = (float)(__bf16)(__uint_as_float(d & 0xffff0000u) * rn);
+          const v2bf y = {(__bf16)(__uint_as_float(g << 16) * h0), (__bf16)(__uint_as_float(g & 0xffff0000u) * h1)};
+          a[it][e] = __builtin_bit_cast(unsigned, y);
+        }
+        if (it * nthr + tid < nchunks) *reinterpret_cast<v4u*>(slot + (size_t)(it * nthr + tid) * 16) = a[it];
+      }
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      asm volatile("s_barrier" ::: "memory");   // the normalized row is complete
+    } else {
+      asm volatile("s_barrier" ::: "memory");
+      // every wave is past its gather of row i - 1: refill that row's slot
+      if (i >= 1 && i - 1 + NS < count)
+        request(x + (size_t)row_of(i + NS - 1) * row_bytes, ((S + NS - 1) % NS) * stride);
+    }
     if (has_block) {
       constexpr int kOff = kImm ? S * 2 * EPL * T : -1;
 #pragma unroll
@@ -638,42 +507,12 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
   if (gamma != nullptr && IS_W) return hipErrorInvalidValue;
   const uint16_t* gm = static_cast<const uint16_t*>(gamma);
   const int threads = ((K >> 5) + 63) & ~63;
-  const uint16_t* xb = static_cast<const uint16_t*>(x);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
   DeviceLimits lim;
   if (hipError_t e = device_limits(&lim); e != hipSuccess) return e;
   hipError_t err = hipSuccess;
-  // R rows interleaved in LDS.  More row groups than `resident` workgroups: each workgroup
-  // streams several groups through a double-buffered tile.
-  auto launch = [&](auto kernel, int R) {
-    const int tile = K * 2 * R;
-    const int ngroups = ceil_div(rows, R);
-    // second LDS buffer: a fixed 16 KB * R behind the first for the 256-lane kernels (see kFixed), else one tile behind
-    const int second = K <= 8192 ? 256 * 64 * R : tile;
-    const int usable = lim.lds_bytes - 1024;   // the kernels' static LDS (row sums of the RMSNorm) stays below 1 KB
-    int per_cu = usable / (second + tile);
-    per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
-    const int resident = lim.cus * per_cu;
-    const bool stream_groups = ngroups > resident && second + tile <= usable;
-    const int grid = stream_groups ? resident : ngroups;
-    const int lds = stream_groups ? second + tile : tile;
-    if (lds > usable) { err = hipErrorInvalidValue; return; }
-    err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), usable);
-    if (err != hipSuccess) return;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), (size_t)lds, stream, xb, idx, rows, K,
-                       KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, stream_groups ? tile : 0, gm, eps);
-    err = hipGetLastError();
-  };
-  constexpr int R = 1;
-  if constexpr (!IS_W) {
-    if (gamma != nullptr) {
-      if (K <= 8192) launch(reorder_quant_kernel<R, false, 256, true>, R);
-      else if (K <= 16384) launch(reorder_quant_kernel<2, false, 512, true>, 2);
-      else launch(reorder_quant_kernel<1, false, 1024, true>, 1);
-      return err;
-    }
-  }
   // rows global -> LDS directly; NS row slots per workgroup, as many workgroups per CU as fit
-  const int usable = lim.lds_bytes - 1024;
+  const int usable = lim.lds_bytes - 1024;   // the kernels' static LDS (row sums of the RMSNorm) stays below 1 KB
   auto launch_dma = [&](auto kernel, int epl, int NS, int nthreads, int max_per_cu) {
     const int lds = NS * 2 * epl * nthreads;   // NS row slots
     if (lds > usable) { err = hipErrorInvalidValue; return; }
@@ -692,8 +531,8 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
     }
     err = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), usable);
     if (err != hipSuccess) return;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(nthreads), (size_t)lds, stream, reinterpret_cast<const uint8_t*>(xb), idx,
-                       rows, K, KN, KS, KO, qn, qs, qo, sfn, sfs, sfo, sched);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(nthreads), (size_t)lds, stream, xb, idx, rows, K, KN, KS, KO, qn, qs, qo, sfn,
+                       sfs, sfo, sched, gm, eps);
     err = hipGetLastError();
   };
   // Measured on M = 4096 ... 16384 rows of K = 3584 ... 18944: two row slots per workgroup, and per CU up to four
@@ -701,42 +540,45 @@ hipError_t launch_reorder_quant(const void* x, const int16_t* idx, int rows, int
   // in front of a workgroup's first row and was slower.
   constexpr int kNS = 2;
   constexpr int kPerCu = 4;
-  // keep: the codes stay in the L2 for the kernel that reads them next (activations only)
-  auto dispatch = [&](auto keep_c) {
+  // keep: the codes stay in the L2 for the kernel that reads them next (activations only); norm: RMSNorm of the row
+  // before the gather (activations only; its codes are always kept: what follows a norm is the layer's GEMM)
+  auto dispatch = [&](auto keep_c, auto norm_c) {
     constexpr bool KP = decltype(keep_c)::value;
+    constexpr bool NM = decltype(norm_c)::value;
     if (K <= 8192) {
       // two lanes per block: K/16 lanes, rounded up to whole waves
       const int t2 = ((K >> 4) + 63) & ~63;
       switch (t2) {
-        case 64: launch_dma(reorder_quant_dma_kernel<16, 64, kNS, IS_W, 64, KP>, 16, kNS, 64, kPerCu); break;
-        case 128: launch_dma(reorder_quant_dma_kernel<16, 128, kNS, IS_W, 128, KP>, 16, kNS, 128, kPerCu); break;
-        case 192: launch_dma(reorder_quant_dma_kernel<16, 192, kNS, IS_W, 192, KP>, 16, kNS, 192, kPerCu); break;
-        case 256: launch_dma(reorder_quant_dma_kernel<16, 256, kNS, IS_W, 256, KP>, 16, kNS, 256, kPerCu); break;
-        case 320: launch_dma(reorder_quant_dma_kernel<16, 320, kNS, IS_W, 320, KP>, 16, kNS, 320, kPerCu); break;
-        case 384: launch_dma(reorder_quant_dma_kernel<16, 384, kNS, IS_W, 384, KP>, 16, kNS, 384, kPerCu); break;
-        case 448: launch_dma(reorder_quant_dma_kernel<16, 448, kNS, IS_W, 448, KP>, 16, kNS, 448, kPerCu); break;
-        default: launch_dma(reorder_quant_dma_kernel<16, 512, kNS, IS_W, 512, KP>, 16, kNS, 512, kPerCu); break;
+        case 64: launch_dma(reorder_quant_dma_kernel<16, 64, kNS, IS_W, 64, KP, NM>, 16, kNS, 64, kPerCu); break;
+        case 128: launch_dma(reorder_quant_dma_kernel<16, 128, kNS, IS_W, 128, KP, NM>, 16, kNS, 128, kPerCu); break;
+        case 192: launch_dma(reorder_quant_dma_kernel<16, 192, kNS, IS_W, 192, KP, NM>, 16, kNS, 192, kPerCu); break;
+        case 256: launch_dma(reorder_quant_dma_kernel<16, 256, kNS, IS_W, 256, KP, NM>, 16, kNS, 256, kPerCu); break;
+        case 320: launch_dma(reorder_quant_dma_kernel<16, 320, kNS, IS_W, 320, KP, NM>, 16, kNS, 320, kPerCu); break;
+        case 384: launch_dma(reorder_quant_dma_kernel<16, 384, kNS, IS_W, 384, KP, NM>, 16, kNS, 384, kPerCu); break;
+        case 448: launch_dma(reorder_quant_dma_kernel<16, 448, kNS, IS_W, 448, KP, NM>, 16, kNS, 448, kPerCu); break;
+        default: launch_dma(reorder_quant_dma_kernel<16, 512, kNS, IS_W, 512, KP, NM>, 16, kNS, 512, kPerCu); break;
       }
     } else if (K <= 20480) {
       // one lane per block: the workgroups are large enough as it is, and LDS (two rows per workgroup) bounds how
       // many a CU holds
       switch (threads) {
-        case 320: launch_dma(reorder_quant_dma_kernel<32, 320, kNS, IS_W, 320, KP>, 32, kNS, 320, kPerCu); break;
-        case 384: launch_dma(reorder_quant_dma_kernel<32, 384, kNS, IS_W, 384, KP>, 32, kNS, 384, kPerCu); break;
-        case 448: launch_dma(reorder_quant_dma_kernel<32, 448, kNS, IS_W, 448, KP>, 32, kNS, 448, kPerCu); break;
-        case 512: launch_dma(reorder_quant_dma_kernel<32, 512, kNS, IS_W, 512, KP>, 32, kNS, 512, kPerCu); break;
-        case 576: launch_dma(reorder_quant_dma_kernel<32, 576, kNS, IS_W, 576, KP>, 32, kNS, 576, kPerCu); break;
-        default: launch_dma(reorder_quant_dma_kernel<32, 640, kNS, IS_W, 640, KP>, 32, kNS, 640, kPerCu); break;
+        case 320: launch_dma(reorder_quant_dma_kernel<32, 320, kNS, IS_W, 320, KP, NM>, 32, kNS, 320, kPerCu); break;
+        case 384: launch_dma(reorder_quant_dma_kernel<32, 384, kNS, IS_W, 384, KP, NM>, 32, kNS, 384, kPerCu); break;
+        case 448: launch_dma(reorder_quant_dma_kernel<32, 448, kNS, IS_W, 448, KP, NM>, 32, kNS, 448, kPerCu); break;
+        case 512: launch_dma(reorder_quant_dma_kernel<32, 512, kNS, IS_W, 512, KP, NM>, 32, kNS, 512, kPerCu); break;
+        case 576: launch_dma(reorder_quant_dma_kernel<32, 576, kNS, IS_W, 576, KP, NM>, 32, kNS, 576, kPerCu); break;
+        default: launch_dma(reorder_quant_dma_kernel<32, 640, kNS, IS_W, 640, KP, NM>, 32, kNS, 640, kPerCu); break;
       }
     } else {
-      launch_dma(reorder_quant_dma_kernel<32, 0, 2, IS_W, 1024, KP>, 32, 2, threads, kPerCu);
+      launch_dma(reorder_quant_dma_kernel<32, 0, 2, IS_W, 1024, KP, NM>, 32, 2, threads, kPerCu);
     }
   };
   if constexpr (IS_W) {
-    dispatch(std::false_type{});
+    dispatch(std::false_type{}, std::false_type{});
   } else {
-    if (keep_codes) dispatch(std::true_type{});
-    else dispatch(std::false_type{});
+    if (gamma != nullptr) dispatch(std::true_type{}, std::true_type{});
+    else if (keep_codes) dispatch(std::true_type{}, std::false_type{});
+    else dispatch(std::false_type{}, std::false_type{});
   }
   return err;
 }

@@ -689,14 +689,27 @@ __device__ __forceinline__ void run_segment(v16f (&acc)[4][TM], HalfFrags<FMT, T
 
 
 // The 0..3 blocks of 32 elements a segment has beyond its whole 128-wide stages (e.g. 4928 = 38 * 128
-// + 64): handled after the pipelined stages, straight from global memory, by two more MFMA steps per
-// segment.  Straight-line code: every load is issued (block index clamped into the segment) and
-// absent blocks are turned into zero codes with scale 2^0 afterwards -- branches around code that
-// touches the accumulator make the register allocator spill it.
+// + 64): straight from global memory, by up to two more MFMA steps per segment (K half h = blocks 2h and
+// 2h + 1), ahead of the pipelined stages.  A half is loaded whole (block index clamped into the segment) and
+// the blocks it does not have are turned into zero codes with scale 2^0 before the MFMAs; a half without any
+// block is skipped by a wave-uniform branch.  Loading and computing are separate steps: the kernel requests the
+// first halves of all three segments before its first stage copies, so that these loads -- 16 bytes per lane from
+// rows far apart, each the first touch of its cache line -- are in flight together and with the copies, and
+// computes them while stages 1 and 2 are still landing.  (After the K loop, one half after the other, they cost
+// 4 to 9 % of the kernel: every load was waited for with nothing else to do; and branches there, around code
+// that touches the live accumulator, make the register allocator spill it.  Here the accumulator is still zero.)
 template <int FMT, int TM>
-__device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][TM], const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
-                                                 const uint8_t* __restrict__ sfa, const uint8_t* __restrict__ sfb, int blk,
-                                                 bool w_tiled, int tiles_n, const Ctx& c) {
+struct RemainderHalf {
+  v4i w[4];
+  typename Fmt<FMT>::xfrag x[TM];
+  int sw[4], sx[TM];
+};
+
+template <int FMT, int TM>
+__device__ __forceinline__ void remainder_load(RemainderHalf<FMT, TM>& f, int h, const uint8_t* __restrict__ a,
+                                               const uint8_t* __restrict__ b, const uint8_t* __restrict__ sfa,
+                                               const uint8_t* __restrict__ sfb, int blk, bool w_tiled, int tiles_n,
+                                               const Ctx& c) {
   const int r = blk & 3, q = blk >> 2;
   // weights: row-major rows of blk blocks, or (tile-major) the r blocks past the whole stages as rows of
   // r blocks behind the tiled part; with r == 0 nothing is used and any valid address will do
@@ -707,54 +720,69 @@ __device__ __forceinline__ void remainder_blocks(v16f (&acc)[4][TM], const uint8
   const int i = c.lane & 31, g = c.lane >> 5;
   const int katoms = (blk + 3) >> 2;
   const unsigned lda = (unsigned)blk * XB;
-  const v4i z = {0, 0, 0, 0};
+  const int kb = 2 * h + g;
+  const int kbc = min(4 * q + kb, blk - 1);           // a block that exists
+  const int kb1 = min(4 * q + 2 * h + 1, blk - 1);    // E4M3: the second block of the half
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int kb = 2 * h + g;
-    const bool ok = kb < r;
-    const int kbc = min(4 * q + kb, blk - 1);           // a block that exists
-    const int kb1 = min(4 * q + 2 * h + 1, blk - 1);    // E4M3: the second block of the half
-    HalfFrags<FMT, TM> f;
-    Scales<TM> sc;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const unsigned n = c.n0 + min(c.wn * 128 + t * 32 + i, c.cols_avail - 1);   // features past the last one are never stored
-      const v4i wv = *reinterpret_cast<const v4i*>(wbase + (size_t)n * wpitch + (size_t)max(kbc - wfirst, 0) * 16);
-      const int sw = sfb[sf_offset(n, kbc, katoms)];
-      f.w[t] = ok ? wv : z;
-      sc.w[t] = ok ? sw : 127;
-    }
-#pragma unroll
-    for (int t = 0; t < TM; ++t) {
-      const unsigned m = c.m0 + min(c.wm * (32 * TM) + t * 32 + i, c.rows_avail - 1);   // rows past the last readable one are never stored
-      const int sx = sfa[sf_offset(m, kbc, katoms)];
-      sc.x[t] = ok ? sx : 127;
-      const uint8_t* xr = a + (size_t)m * lda;
-      if constexpr (FMT == kFmtE2M1) {
-        const v4i xv = *reinterpret_cast<const v4i*>(xr + (size_t)kbc * 16);
-        f.x[t] = ok ? xv : z;
-      } else if constexpr (FMT == kFmtE3M2) {
-        const v2i* p = reinterpret_cast<const v2i*>(xr + (size_t)kbc * 24);
-        const v2i p0 = p[0], p1 = p[1], p2 = p[2];
-        const v6i xv = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1]};
-        const v6i z6 = {0, 0, 0, 0, 0, 0};
-        f.x[t] = ok ? xv : z6;
-      } else {
-        // K [16g, 16g+16) of the half lies in block 2h, K [32+16g, ...) in block 2h+1
-        const int kb0 = min(4 * q + 2 * h, blk - 1);
-        const v4i pa = *reinterpret_cast<const v4i*>(xr + (size_t)kb0 * 32 + g * 16);
-        const v4i pb = *reinterpret_cast<const v4i*>(xr + (size_t)kb1 * 32 + g * 16);
-        const v4i va = 2 * h < r ? pa : z, vb = 2 * h + 1 < r ? pb : z;
-        f.x[t] = __builtin_shufflevector(va, vb, 0, 1, 2, 3, 4, 5, 6, 7);
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int tn = 0; tn < 4; ++tn)
-#pragma unroll
-      for (int tm = 0; tm < TM; ++tm) mfma_one<FMT, 0>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
-    __builtin_amdgcn_sched_barrier(0);
+  for (int t = 0; t < 4; ++t) {
+    const unsigned n = c.n0 + min(c.wn * 128 + t * 32 + i, c.cols_avail - 1);   // features past the last one are never stored
+    f.w[t] = *reinterpret_cast<const v4i*>(wbase + (size_t)n * wpitch + (size_t)max(kbc - wfirst, 0) * 16);
+    f.sw[t] = sfb[sf_offset(n, kbc, katoms)];
   }
+#pragma unroll
+  for (int t = 0; t < TM; ++t) {
+    const unsigned m = c.m0 + min(c.wm * (32 * TM) + t * 32 + i, c.rows_avail - 1);   // rows past the last readable one are never stored
+    f.sx[t] = sfa[sf_offset(m, kbc, katoms)];
+    const uint8_t* xr = a + (size_t)m * lda;
+    if constexpr (FMT == kFmtE2M1) {
+      f.x[t] = *reinterpret_cast<const v4i*>(xr + (size_t)kbc * 16);
+    } else if constexpr (FMT == kFmtE3M2) {
+      const v2i* p = reinterpret_cast<const v2i*>(xr + (size_t)kbc * 24);
+      const v2i p0 = p[0], p1 = p[1], p2 = p[2];
+      f.x[t] = v6i{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1]};
+    } else {
+      // K [16g, 16g+16) of the half lies in block 2h, K [32+16g, ...) in block 2h+1
+      const int kb0 = min(4 * q + 2 * h, blk - 1);
+      const v4i pa = *reinterpret_cast<const v4i*>(xr + (size_t)kb0 * 32 + g * 16);
+      const v4i pb = *reinterpret_cast<const v4i*>(xr + (size_t)kb1 * 32 + g * 16);
+      f.x[t] = __builtin_shufflevector(pa, pb, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  }
+}
+
+template <int FMT, int TM>
+__device__ __forceinline__ void remainder_mfma(v16f (&acc)[4][TM], RemainderHalf<FMT, TM>& f, int h, int blk, const Ctx& c) {
+  const int r = blk & 3;
+  const int g = c.lane >> 5;
+  const bool ok = 2 * h + g < r;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f.w[t][e] = ok ? f.w[t][e] : 0;
+    f.sw[t] = ok ? f.sw[t] : 127;
+  }
+#pragma unroll
+  for (int t = 0; t < TM; ++t) {
+    f.sx[t] = ok ? f.sx[t] : 127;
+    if constexpr (FMT == kFmtE4M3) {
+      const bool oka = 2 * h < r, okb = 2 * h + 1 < r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        f.x[t][e] = oka ? f.x[t][e] : 0;
+        f.x[t][4 + e] = okb ? f.x[t][4 + e] : 0;
+      }
+    } else {
+      constexpr int NE = FMT == kFmtE2M1 ? 4 : 6;
+#pragma unroll
+      for (int e = 0; e < NE; ++e) f.x[t][e] = ok ? f.x[t][e] : 0;
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) mfma_one<FMT, 0>(acc[tn][tm], f.w[tn], f.x[tm], f.sw[tn], f.sx[tm]);
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 // REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
@@ -834,6 +862,16 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   const LaneOffsets lo(plan, c);
   const WeightPtrs wp(lds, c, TM);
 
+  // the blocks past the whole stages first (see RemainderHalf): first K halves requested ahead of the copies
+  RemainderHalf<kFmtE2M1, TM> p0;
+  RemainderHalf<kFmtE3M2, TM> s0;
+  RemainderHalf<kFmtE4M3, TM> o0;
+  if constexpr (REM) {
+    if ((plan.blk0 & 3) > 0) remainder_load<kFmtE2M1>(p0, 0, plan.a0, plan.b0, plan.sfa0, plan.sfb0, plan.blk0, WT, tiles_n, c);
+    if ((plan.blk1 & 3) > 0) remainder_load<kFmtE3M2>(s0, 0, plan.a1, plan.b1, plan.sfa1, plan.sfb1, plan.blk1, WT, tiles_n, c);
+    if ((plan.blk2 & 3) > 0) remainder_load<kFmtE4M3>(o0, 0, plan.a2, plan.b2, plan.sfa2, plan.sfb2, plan.blk2, WT, tiles_n, c);
+    __builtin_amdgcn_sched_barrier(0);
+  }
   // prologue: stages 0 and 1 and the first copies of stage 2 in flight; wait for stage 0 only.  The copies go out
   // before anything else that can wait (the accumulators are cleared while they are in flight); in REGULAR kernels
   // the first three stages are E2M1 stages, or do not exist, and take the compile-time form of the copies.
@@ -883,6 +921,24 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
   __builtin_amdgcn_sched_barrier(0);
 
+  if constexpr (REM) {
+    if ((plan.blk0 & 3) > 0) remainder_mfma<kFmtE2M1>(acc, p0, 0, plan.blk0, c);
+    if ((plan.blk1 & 3) > 0) remainder_mfma<kFmtE3M2>(acc, s0, 0, plan.blk1, c);
+    if ((plan.blk2 & 3) > 0) remainder_mfma<kFmtE4M3>(acc, o0, 0, plan.blk2, c);
+    // second K halves: segments with three blocks past their whole stages
+    RemainderHalf<kFmtE2M1, TM> p1;
+    RemainderHalf<kFmtE3M2, TM> s1;
+    RemainderHalf<kFmtE4M3, TM> o1;
+    if ((plan.blk0 & 3) > 2) remainder_load<kFmtE2M1>(p1, 1, plan.a0, plan.b0, plan.sfa0, plan.sfb0, plan.blk0, WT, tiles_n, c);
+    if ((plan.blk1 & 3) > 2) remainder_load<kFmtE3M2>(s1, 1, plan.a1, plan.b1, plan.sfa1, plan.sfb1, plan.blk1, WT, tiles_n, c);
+    if ((plan.blk2 & 3) > 2) remainder_load<kFmtE4M3>(o1, 1, plan.a2, plan.b2, plan.sfa2, plan.sfb2, plan.blk2, WT, tiles_n, c);
+    __builtin_amdgcn_sched_barrier(0);
+    if ((plan.blk0 & 3) > 2) remainder_mfma<kFmtE2M1>(acc, p1, 1, plan.blk0, c);
+    if ((plan.blk1 & 3) > 2) remainder_mfma<kFmtE3M2>(acc, s1, 1, plan.blk1, c);
+    if ((plan.blk2 & 3) > 2) remainder_mfma<kFmtE4M3>(acc, o1, 1, plan.blk2, c);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
   wait_copies_but(in_flight);
   asm volatile("s_barrier" ::: "memory");
 
@@ -912,14 +968,6 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
     run_segment<kFmtE3M2, kFmtNone, kFmtE3M2, REGULAR, NLAST>(acc, a6, sc, none6, l6, l0, gc, lo, plan, n6, 0, n4, wp, lds, c);
   } else {
     run_segment<kFmtE2M1, kFmtNone, kFmtE2M1, REGULAR>(acc, a4, sc, none4, l4, l0, gc, lo, plan, n4, 0, 0, wp, lds, c);
-  }
-
-  if constexpr (REM) {
-    __builtin_amdgcn_sched_barrier(0);
-    remainder_blocks<kFmtE2M1>(acc, plan.a0, plan.b0, plan.sfa0, plan.sfb0, plan.blk0, WT, tiles_n, c);
-    remainder_blocks<kFmtE3M2>(acc, plan.a1, plan.b1, plan.sfa1, plan.sfb1, plan.blk1, WT, tiles_n, c);
-    remainder_blocks<kFmtE4M3>(acc, plan.a2, plan.b2, plan.sfa2, plan.sfb2, plan.blk2, WT, tiles_n, c);
-    __builtin_amdgcn_sched_barrier(0);
   }
 
   // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.

@@ -237,6 +237,9 @@ BIG_TILE_SHAPES = [
     (2304, 3840, 384, 384, 128), (2304, 3840, 384, 384, 256), (2304, 3840, 384, 384, 384), (2304, 3840, 448, 416, 224),
     (2304, 3840, 512, 0, 0), (2304, 3840, 384, 128, 0), (2304, 3840, 384, 256, 0), (2304, 3840, 384, 0, 128),
     (2304, 3840, 384, 0, 384), (2100, 3848, 384, 384, 128),
+    # 1, 2 and 3 blocks of 32 past the whole stages in every segment (computed ahead of the K loop, absent K halves
+    # skipped), with and without compiled-in segment boundaries, ragged tokens and features
+    (2304, 3840, 416, 480, 160), (2304, 3840, 480, 448, 192), (2304, 3840, 160, 224, 352), (2100, 3848, 480, 448, 192),
 ]
 
 

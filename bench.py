@@ -101,10 +101,17 @@ def event_ms(pairs):
     return sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
 
 
-def graph_ms(launch, iters, warmup=3, repeats=3):
-    """Average time of one launch when `iters` back-to-back launches (launch(i), i = 0..iters-1, no
+GRAPH_WARM_S = 0.15   # untimed replays in front of a graph measurement (0 with --no-clock-warmup)
+
+
+def graph_ms(launch, iters, warmup=3, repeats=5):
+    """Time of one launch when `iters` back-to-back launches (launch(i), i = 0..iters-1, no
     allocation inside) are replayed as one HIP graph: the host's per-call cost (10-15 us through ctypes)
-    is out of the measurement, which a 10 us kernel needs.  Mean over `repeats` replays."""
+    is out of the measurement, which a 10 us kernel needs.  The graph is first replayed untimed for
+    GRAPH_WARM_S seconds (after the host-side set-up of a leg the GPU has idled and runs the first
+    milliseconds at other clocks, as the headline's warm-up steps account for); then the median over
+    `repeats` timed replays."""
+    import time
     import torch
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -119,19 +126,25 @@ def graph_ms(launch, iters, warmup=3, repeats=3):
     torch.cuda.synchronize()
     g.replay()
     torch.cuda.synchronize()
-    total = 0.0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < GRAPH_WARM_S:
+        for _ in range(4):
+            g.replay()
+        torch.cuda.synchronize()
+    times = []
     for _ in range(repeats):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         g.replay()
         e1.record()
         torch.cuda.synchronize()
-        total += e0.elapsed_time(e1)
+        times.append(e0.elapsed_time(e1))
     del g
-    return total / (repeats * iters)
+    return sorted(times)[len(times) // 2] / iters
 
 
 def main():
+    global GRAPH_WARM_S
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
@@ -208,6 +221,8 @@ def main():
     # than the steady state, and the counted warm-up may be a handful of steps.
     t_warm = time.perf_counter()
     warm_steps = 0
+    if args.no_clock_warmup:
+        GRAPH_WARM_S = 0.0
     while time.perf_counter() - t_warm < (0.0 if args.no_clock_warmup else 0.4):
         for _ in range(20):
             step()
@@ -455,7 +470,7 @@ def main():
                            "quant_gbs": round(quant_bytes(mm, kk, knm, ksm, kom) / (times[0] * 1e-3) / 1e9, 1)})
             del xm, wqm, aqm, dm
         extra["shape_matrix"] = {"note": "back-to-back launches on one buffer set (operands may sit in the 256 MB "
-                                         "Infinity Cache); 20 launches per kernel replayed as a HIP graph, 3 replays", "rows": matrix}
+                                         "Infinity Cache); 20 launches per kernel replayed as a HIP graph: 0.15 s of untimed replays, then the median of 5", "rows": matrix}
 
         # ------------------------------------------------------------ one activation format at a time (c3's M, N, K)
         # the 256x256 kernel needs all three segments, so the other two get one 128-wide stage each

@@ -785,23 +785,40 @@ __device__ __forceinline__ void remainder_mfma(v16f (&acc)[4][TM], RemainderHalf
   __builtin_amdgcn_sched_barrier(0);
 }
 
-// REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
-// SEGS: which activation segments the plan has, bit 0 E2M1 (always), bit 1 E3M2, bit 2 E4M3 -- the
-// prefetched fragments pass from a segment to the next one that exists, and their types are fixed here.
-// TM: token tiles of 32 per wave.  4: the workgroup's tile is 256 features x 256 tokens.  2: 256 x 128, for
-// problems with fewer than 256 whole tiles (every CU still gets a workgroup): same copies (the lanes of token
-// rows 128 ... 255 read the last row again, which costs the address unit next to nothing), same LDS image,
-// half the MFMAs per stage, a copy slot after every MFMA instead of every second one.
-// NLAST: see run_segment (the launcher picks the instance from the plan).
-template <bool REGULAR, bool REM, bool WT, int SEGS = 7, int TM = 4, int NLAST = 0>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d, int first_round,
-                      int skew) {
-  extern __shared__ __align__(16) uint8_t lds[];
-  // Staggered start: with several tiles per CU, the first workgroup of each CU (the first `first_round` of the
-  // grid) starts up to `skew` clock ticks late, each by a different amount.  Every tile takes the same time, so
-  // without this all CUs load their first stages and store their result tiles in the same microseconds, tile after
-  // tile, and queue at the memory; the few microseconds lost once come back several times over.
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give each XCD a contiguous band of
+// feature tiles and walk it feature tile by feature tile inside groups of at most 8 feature tiles, token tile
+// after token tile: the ~32 tiles an XCD works on at a time are then about as many feature tiles as token tiles
+// (7 x 4.6 for 56 x 16 tiles), which is what keeps the bytes that pass its L2 lowest.
+__device__ __forceinline__ void tile_of(int wg, int nwg, int tiles_n, int& tile_n, int& tile_m) {
+  const int tiles_m = nwg / tiles_n;
+  tile_n = wg / tiles_m;
+  tile_m = wg % tiles_m;
+  if ((nwg & 7) == 0) {
+    const int per_xcd = nwg >> 3;
+    const int j = wg >> 3;                       // position in this XCD's list
+    const int tile = (wg & 7) * per_xcd + j;     // feature-major tile index
+    tile_n = tile / tiles_m;
+    tile_m = tile % tiles_m;
+    if (per_xcd % tiles_m == 0) {
+      const int cols = per_xcd / tiles_m;        // feature tiles of the band
+      const int groups = (cols + 7) / 8;
+      if (cols % groups == 0) {
+        const int gw = cols / groups, per_group = gw * tiles_m;
+        const int g = j / per_group, r = j % per_group;
+        tile_n = (wg & 7) * cols + g * gw + r % gw;
+        tile_m = r / gw;
+      }
+    }
+  }
+}
+
+// What a workgroup does before its tile: the staggered start and the plan into scalar registers.
+// Staggered start: with several tiles per CU, the first workgroup of each CU (the first `first_round` of the
+// grid) starts up to `skew` clock ticks late, each by a different amount.  Every tile takes the same time, so
+// without this all CUs load their first stages and store their result tiles in the same microseconds, tile after
+// tile, and queue at the memory; the few microseconds lost once come back several times over.
+template <bool WT>
+__device__ __forceinline__ Plan start_workgroup(const Plan& plan_arg, int first_round, int skew) {
   if (skew > 0 && (int)blockIdx.x < first_round) {
     const long long delay = (long long)skew * (((int)blockIdx.x >> 3) * 8 + ((int)blockIdx.x & 7)) / first_round;
     const long long t0 = __builtin_amdgcn_s_memtime();
@@ -820,37 +837,27 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   plan.blk2 = __builtin_amdgcn_readfirstlane(plan_arg.blk2);
   plan.total = __builtin_amdgcn_readfirstlane(plan_arg.total);
   plan.w_tiled = WT ? 1 : 0;
+  return plan;
+}
 
+// REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
+// SEGS: which activation segments the plan has, bit 0 E2M1 (always), bit 1 E3M2, bit 2 E4M3 -- the
+// prefetched fragments pass from a segment to the next one that exists, and their types are fixed here.
+// TM: token tiles of 32 per wave.  4: the workgroup's tile is 256 features x 256 tokens.  2: 256 x 128, for
+// problems with fewer than 256 whole tiles (every CU still gets a workgroup): same copies (the lanes of token
+// rows 128 ... 255 read the last row again, which costs the address unit next to nothing), same LDS image,
+// half the MFMAs per stage, a copy slot after every MFMA instead of every second one.
+// NLAST: see run_segment (the launcher picks the instance from the plan).
+// Computes one tile of 256 features x 64 * TM tokens: feature tile tile_n, token tile tile_m (of 64 * TM rows).
+template <bool REGULAR, bool REM, bool WT, int SEGS, int TM, int NLAST>
+__device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int tile_m, int tiles_n, int N, int m_store,
+                                             int a_rows, uint16_t* __restrict__ d, uint8_t* lds) {
   const int tid = threadIdx.x;
   Ctx c;
   c.lane = tid & 63;
   c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   c.wn = c.wave & 1;
   c.wm = c.wave >> 1;
-  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give each XCD a contiguous band of
-  // feature tiles and walk it feature tile by feature tile inside groups of at most 8 feature tiles, token tile
-  // after token tile: the ~32 tiles an XCD works on at a time are then about as many feature tiles as token tiles
-  // (7 x 4.6 for 56 x 16 tiles), which is what keeps the bytes that pass its L2 lowest.
-  const int wg = blockIdx.x, nwg = gridDim.x;
-  const int tiles_m = nwg / tiles_n;
-  int tile_n = wg / tiles_m, tile_m = wg % tiles_m;
-  if ((nwg & 7) == 0) {
-    const int per_xcd = nwg >> 3;
-    const int j = wg >> 3;                       // position in this XCD's list
-    int tile = (wg & 7) * per_xcd + j;           // feature-major tile index
-    tile_n = tile / tiles_m;
-    tile_m = tile % tiles_m;
-    if (per_xcd % tiles_m == 0) {
-      const int cols = per_xcd / tiles_m;        // feature tiles of the band
-      const int groups = (cols + 7) / 8;
-      if (cols % groups == 0) {
-        const int gw = cols / groups, per_group = gw * tiles_m;
-        const int g = j / per_group, r = j % per_group;
-        tile_n = (wg & 7) * cols + g * gw + r % gw;
-        tile_m = r / gw;
-      }
-    }
-  }
   constexpr int kTokens = 64 * TM;   // token rows of the workgroup's tile
   c.n0 = tile_n * kT;
   c.m0 = tile_m * kTokens;
@@ -1022,6 +1029,43 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   }
 }
 
+
+template <bool REGULAR, bool REM, bool WT, int SEGS = 7, int TM = 4, int NLAST = 0>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d, int first_round,
+                      int skew) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const Plan plan = start_workgroup<WT>(plan_arg, first_round, skew);
+  int tile_n, tile_m;
+  tile_of(blockIdx.x, gridDim.x, tiles_n, tile_n, tile_m);
+  compute_tile<REGULAR, REM, WT, SEGS, TM, NLAST>(plan, tile_n, tile_m, tiles_n, N, m_store, a_rows, d, lds);
+}
+
+// The same for problems whose last round of 256 x 256 tiles would leave at least half of the CUs idle: the first
+// n_whole workgroups compute whole tiles (n_whole a multiple of the CU count), the others the remaining whole tiles
+// as two tiles of 256 x 128 each.  A half tile takes about 0.7 of a whole tile's time, and the half-empty round took
+// as long as a full one (M = 3072 and 4096 at N = 14336, K = 4096: 768 tiles 101.5 us, 896 tiles 134.1 us).
+template <bool REM, bool WT, int NLAST>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+mixed_gemm_256_tail_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d, int first_round,
+                           int skew, int n_whole) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const Plan plan = start_workgroup<WT>(plan_arg, first_round, skew);
+  const int wg = blockIdx.x;
+  const int ntiles = n_whole + (((int)gridDim.x - n_whole) >> 1);   // whole tiles of the problem
+  int tile_n, tile_m;
+  if (wg < n_whole) {
+    tile_of(wg, ntiles, tiles_n, tile_n, tile_m);
+    compute_tile<true, REM, WT, 7, 4, NLAST>(plan, tile_n, tile_m, tiles_n, N, m_store, a_rows, d, lds);
+  } else {
+    const int h = wg - n_whole;
+    tile_of(n_whole + (h >> 1), ntiles, tiles_n, tile_n, tile_m);
+    const int half_m = 2 * tile_m + (h & 1);
+    if (half_m * 128 >= m_store) return;   // the lower half of a ragged last tile: no token of it exists
+    compute_tile<true, REM, WT, 7, 2, NLAST>(plan, tile_n, half_m, tiles_n, N, m_store, a_rows, d, lds);
+  }
+}
+
 }  // namespace
 
 
@@ -1073,6 +1117,14 @@ static kernel_t select_kernel(bool regular, int segs, int nlast) {
   return nullptr;
 }
 
+typedef void (*tail_kernel_t)(Plan, int, int, int, int, uint16_t*, int, int, int);
+
+template <bool REM, bool WT>
+static tail_kernel_t select_tail_kernel(int nlast) {
+  return nlast == 1 ? mixed_gemm_256_tail_kernel<REM, WT, 1>
+                    : (nlast == 2 ? mixed_gemm_256_tail_kernel<REM, WT, 2> : mixed_gemm_256_tail_kernel<REM, WT, 3>);
+}
+
 hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, const uint8_t* bs,
                                  const uint8_t* ao, const uint8_t* bo, const uint8_t* sfan, const uint8_t* sfbn,
                                  const uint8_t* sfas, const uint8_t* sfbs, const uint8_t* sfao, const uint8_t* sfbo,
@@ -1101,6 +1153,16 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
     else kernel = half ? select_kernel<false, false, 2>(regular, segs, nlast) : select_kernel<false, false, 4>(regular, segs, nlast);
   }
   if (kernel == nullptr) return hipErrorInvalidValue;
+  // a last round of whole tiles on at most half of the CUs: those tiles as twice as many half tiles
+  const int whole_tiles = ((N + kT - 1) / kT) * (M / tokens);
+  const int rest = whole_tiles % lim.cus;
+  const bool tail = !half && regular && segs == 7 && whole_tiles > lim.cus && rest > 0 && 2 * rest <= lim.cus;
+  tail_kernel_t tail_kernel = nullptr;
+  if (tail) {
+    if (rem) tail_kernel = w_tiled ? select_tail_kernel<true, true>(nlast) : select_tail_kernel<true, false>(nlast);
+    else tail_kernel = w_tiled ? select_tail_kernel<false, true>(nlast) : select_tail_kernel<false, false>(nlast);
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(tail_kernel), kBuffers * kStage); e != hipSuccess) return e;
+  }
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kBuffers * kStage); e != hipSuccess) return e;
   Plan p;
   p.a0 = an; p.a1 = as_; p.a2 = ao;
@@ -1116,8 +1178,12 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   // more tiles than CUs: staggered start (see the kernel), up to kStartSkew ticks of the shader's clock counter
   const int ntiles = tiles_n * tiles_m;
   const int skew = ntiles > lim.cus ? kStartSkew : 0;
-  hipLaunchKernelGGL(kernel, dim3(ntiles), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,
-                     static_cast<uint16_t*>(d), lim.cus, skew);
+  if (tail)
+    hipLaunchKernelGGL(tail_kernel, dim3(ntiles + rest), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,
+                       static_cast<uint16_t*>(d), lim.cus, skew, ntiles - rest);
+  else
+    hipLaunchKernelGGL(kernel, dim3(ntiles), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,
+                       static_cast<uint16_t*>(d), lim.cus, skew);
   return hipGetLastError();
 }
 

@@ -240,6 +240,11 @@ BIG_TILE_SHAPES = [
     # 1, 2 and 3 blocks of 32 past the whole stages in every segment (computed ahead of the K loop, absent K halves
     # skipped), with and without compiled-in segment boundaries, ragged tokens and features
     (2304, 3840, 416, 480, 160), (2304, 3840, 480, 448, 192), (2304, 3840, 160, 224, 352), (2100, 3848, 480, 448, 192),
+    # more whole tiles than CUs with a last round on at most half of them: those tiles run as half tiles in the same
+    # launch (272 = 256 + 16 tiles; a last segment of 1, 2, 3 stages; blocks past the whole stages; ragged tokens whose
+    # last tile has no lower half; features that are not whole tiles)
+    (4352, 4096, 384, 384, 128), (4352, 4096, 384, 384, 256), (4352, 4096, 384, 384, 384), (4352, 4096, 448, 416, 224),
+    (4200, 4096, 384, 384, 128), (4300, 4104, 448, 416, 224),
 ]
 
 

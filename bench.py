@@ -318,9 +318,9 @@ def main():
         zw = abi.reorder_quantize_w(torch.zeros_like(wd), idd, kn, ks, ko)
         zb = abi.tile_weights(*zw[:3])
         zr, rr = [], []
-        for it in range(5):
+        for _ in range(5):   # straight after the leg above: the GPU has not idled
             zr.append(graph_ms(lambda i: abi.matmul(zq[0], zb[0], zq[1], zb[1], zq[2], zb[2], zq[3], zw[3], zq[4], zw[4],
-                                                    zq[5], zw[5], out=d, w_tiled=True), 20, repeats=2, warm_s=None if it == 0 else 0.0))
+                                                    zq[5], zw[5], out=d, w_tiled=True), 20, repeats=2, warm_s=0.0))
             rr.append(graph_ms(lambda i: abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4],
                                                     aq[5], bq[5], out=d, w_tiled=True), 20, repeats=2, warm_s=0.0))
         z_ms, r_ms = sorted(zr)[2], sorted(rr)[2]

@@ -689,12 +689,30 @@ static bool decode_lds_plan(const DecodeSeg& d4, const DecodeSeg& d6, const Deco
   return pos <= 76 * 1024;
 }
 
-// Feature groups of 16 per workgroup of the skinny kernel.
+// Feature groups of 16 per workgroup of the decode kernel (and what the cost model below assumes of the skinny one).
 static int skinny_feature_groups(int rows, int N, int cus) {
   const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
   return ceil_div(N, 32) * ceil_div(rows, 16 * g) >= cus ? 2 : 1;
 }
 
+// Token groups (g) and feature groups (f) of 16 per workgroup of the skinny kernel.  A wave's loads per K step are
+// f weight fragments, 2 g token fragments and f + g scale bytes, and the token fragments (16 rows x 16 bytes each)
+// are what the address unit is slowest at: two feature groups per workgroup halve them per output, and more than
+// four token groups per workgroup never paid (M = 128, N = 4096, K = 4096: g = 8, f = 1 22.3 us; g = 4, f = 2 16.9 us;
+// M = 64: g = 4, f = 1 12.0 us; g = 2, f = 2 10.5 us; M = 200: g = 8, f = 2 26.4 us; g = 4, f = 2 23.0 us).  The largest of
+// these that still gives every CU a workgroup.
+static void skinny_groups(int rows, int N, int cus, int* g_out, int* f_out) {
+  const int gmax = rows <= 16 ? 1 : (rows <= 32 ? 2 : 4);
+  for (int f = 2; f >= 1; --f)
+    for (int g = gmax; g >= 1; g >>= 1)
+      if (ceil_div(N, 16 * f) * ceil_div(rows, 16 * g) >= cus) {
+        *g_out = g;
+        *f_out = f;
+        return;
+      }
+  *g_out = 1;
+  *f_out = 1;
+}
 hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int N,
                          bool w_tiled, uint16_t* d, hipStream_t stream) {
   const int rows = M;
@@ -725,11 +743,8 @@ hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeS
     }
   }
   const int steps_per_wave = (d4.steps + d6.steps + d8.steps + 3) / 4;
-  const int g = rows <= 16 ? 1 : (rows <= 32 ? 2 : (rows <= 64 ? 4 : 8));
-  // two feature groups per workgroup for 17-64 tokens: each activation fragment then serves 32 features
-  // two feature groups per workgroup (an activation fragment then serves 32 features) as long as that
-  // leaves a workgroup for every CU; measured on N = 2048 ... 14336
-  const int f = skinny_feature_groups(rows, N, lim.cus);
+  int g, f;
+  skinny_groups(rows, N, lim.cus, &g, &f);
   const dim3 grid(ceil_div(N, 16 * f), ceil_div(rows, 16 * g));
   const int wt = w_tiled ? 1 : 0;
   switch (g) {
@@ -1046,17 +1061,20 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
                                  int m_store, int a_rows, int N, int KN, int KS, int KO, bool w_tiled, void* d,
                                  hipStream_t stream);
 
-// Rough launch times in microseconds (measured on MI355X, K = 4096: a 128-wide stage takes ~1.05 us
-// with every CU busy and ~0.7 us when at most half of them are, plus ~8 us of fill and drain per
-// round of 256 tiles; 0.19-0.25 ns per 16 tokens x 16 features x 128 K on the skinny kernel), only to
-// choose between the two for fewer than 256 tokens.
-static double pipelined_us(int m_pad, int N, int stages) {
-  const int tiles = (m_pad / 256) * ((N + 255) / 256);
-  return (double)((tiles + 255) / 256) * (stages * (tiles <= 128 ? 0.7 : 1.05) + 8.0);
+// Rough launch times in microseconds, only to choose between the two kernels for fewer than 256 tokens (measured on
+// MI355X, 256 CUs, K = 4096: the whole-tile kernel runs such problems as 256 x 128 tiles when that is at most one
+// round -- a 128-wide stage then takes ~0.5 us with at most half of the CUs busy, ~0.6 us with more, plus ~2.5 us --
+// and as 256 x 256 tiles at ~1.05 us a stage plus ~3 us a round otherwise; the skinny kernel takes 0.18-0.25 ns per
+// 16 tokens x 16 features x 128 K plus ~5 us).
+static double pipelined_us(int M, int N, int stages, int cus) {
+  const int whole = ceil_div(M, 256) * ceil_div(N, 256);
+  if (whole <= cus / 2) return stages * (ceil_div(M, 128) * ceil_div(N, 256) <= cus / 2 ? 0.5 : 0.6) + 2.5;
+  return (double)ceil_div(whole, cus) * (stages * 1.05 + 3.0);
 }
-static double skinny_us(int rows, int N, int steps) {
-  const double per_unit = skinny_feature_groups(rows, N, 256) == 2 ? 0.19e-3 : 0.25e-3;   // (the figures are MI355X's: 256 CUs)
-  return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * per_unit;
+static double skinny_us(int rows, int N, int steps, int cus) {
+  int g, f;
+  skinny_groups(rows, N, cus, &g, &f);
+  return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * (f == 2 ? 0.18e-3 : 0.25e-3);
 }
 
 // a_rows: token rows for which the activation codes and scales are readable (>= M)
@@ -1070,10 +1088,16 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
   if (w_tiled && (N % 256 != 0 || !mixed_gemm_256_supported(256, N, KN, KS, KO))) return hipErrorInvalidValue;
   const int m_pad = (M + 255) / 256 * 256;
   const int steps = (KN + 127) / 128 + (KS + 127) / 128 + (KO + 127) / 128;
+  int cus = 256;
+  if (M < 256) {
+    DeviceLimits lim;
+    if (hipError_t e = device_limits(&lim); e != hipSuccess) return e;
+    cus = lim.cus;
+  }
   // whole 256-row tiles; the last one does not write rows past M and reads no activation row past
   // a_rows (lanes that would are pointed at the last readable row)
   if (mixed_gemm_256_supported(m_pad, N, KN, KS, KO) &&
-      (M >= 256 || pipelined_us(m_pad, N, steps) < skinny_us(M, N, steps)))
+      (M >= 256 || pipelined_us(M, N, steps, cus) < skinny_us(M, N, steps, cus)))
     return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, a_rows, N, KN, KS, KO,
                                  w_tiled, d, stream);
   const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};

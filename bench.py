@@ -41,7 +41,7 @@ MEASURED_TRAFFIC = {
     "quant_c1": {"bytes": int((16465.5 * 1.99980 + 10517.6 * 1.0) * 1024),       # 44.5 MB against 44.2 MB algorithmic
                  "source": "mixedgemm_amd/csrc/reorder_quant.hip", "sha": "1d89b7fe0d03a81d"},
     "decode_c2": {"bytes": int((16318.0 * 1.99980 + 896.0 * 1.0) * 1024),        # 34.3 MB against 31.4 MB algorithmic (tile-major weights)
-                  "source": "mixedgemm_amd/csrc/mixed_gemm.hip", "sha": "ad3adce2dd250e7c"},
+                  "source": "mixedgemm_amd/csrc/mixed_gemm.hip", "sha": "a6cdb0f27150abfe"},
     "calibrate_c1": {"bytes": int(((16411.0 + 1045.0 + 81.5) * 1.99980 + (2048.0 + 16.0 + 56.2) * 1.0) * 1024),   # three kernels
                      "source": "mixedgemm_amd/csrc/calibrate.hip", "sha": "84a260f8dfd73ec0"},
 }

@@ -139,7 +139,7 @@ mixed_gemm_direct_kernel(const uint8_t* __restrict__ an, const uint8_t* __restri
 // Skinny kernel: few tokens (decode, small batches), weights streamed once per
 // 16 * G tokens (HBM- or L2-bound).
 //
-// A workgroup of 4 waves owns 16 output features and G groups of 16 tokens; the K
+// A workgroup of 4 waves owns F groups of 16 output features and G groups of 16 tokens; the K
 // steps (128 elements each, counted over the three segments) are dealt to the 4
 // waves in contiguous quarters.  A wave issues every load of a round of steps
 // (weights, the G token groups, scales; addresses clamped, no branches) before
@@ -756,13 +756,9 @@ hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeS
       if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<2, 2>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
       else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<2, 1>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
       break;
-    case 4:
+    default:   // 4 token groups: skinny_groups takes no more
       if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<4, 2>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
       else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<4, 1>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
-      break;
-    default:
-      if (f == 2) hipLaunchKernelGGL((mixed_gemm_skinny_kernel<8, 2>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
-      else hipLaunchKernelGGL((mixed_gemm_skinny_kernel<8, 1>), grid, dim3(256), 0, stream, d4, d6, d8, M, N, steps_per_wave, wt, d);
       break;
   }
   return hipGetLastError();

@@ -550,6 +550,40 @@ def test_tiled_weights_give_the_same_result_bit_for_bit(abi, m, n, kn, ks, ko):
     _check_gemm(d3, qx, qw, "tiled, exact-size buffers")
 
 
+@pytest.mark.parametrize("m,m_part,n,kn,ks,ko", [
+    # 272 whole tiles: 256 + 16 run as 32 half tiles; the first 4096 rows alone are 256 whole tiles, one round
+    (4352, 4096, 4096, 384, 384, 128), (4352, 4096, 4096, 448, 416, 224), (4200, 4096, 4096, 384, 384, 384),
+    # 144 whole tiles against 128 (at most half of the CUs: all of them as half tiles)
+    (2304, 2048, 4096, 480, 448, 192),
+])
+def test_mixed_tile_heights_equal_the_plain_launch_bit_for_bit(abi, m, m_part, n, kn, ks, ko):
+    """A launch that runs its last round (or all of its tiles) as 256 x 128 tiles adds the same products in the same
+    order per output element as one that runs 256 x 256 tiles: the rows the two have in common are equal bit for
+    bit.  The part call sees the first m_part token rows only (code rows and scale atoms are prefixes)."""
+    _say("mixed tile heights", m, m_part, n, kn, ks, ko)
+    k = kn + ks + ko
+    x = H.make_activations(m, k, 71 + m + n, n_out=max(1, k // 32))
+    w = H.make_weights(n, k, 73 + m + n)
+    idx = H.absmax_sort_index(x)
+    xd, wd, idd = x.to(DEV), w.to(DEV), idx.to(DEV)
+    bq = abi.reorder_quantize_w(wd, idd, kn, ks, ko)
+    if abi.weights_tileable(n, kn, ks, ko):
+        bq = abi.tile_weights(*bq[:3]) + bq[3:]
+        tiled = True
+    else:
+        tiled = False
+    aq = abi.reorder_quantize_x(xd, idd, kn, ks, ko)
+    full = abi.matmul(aq[0], bq[0], aq[1], bq[1], aq[2], bq[2], aq[3], bq[3], aq[4], bq[4], aq[5], bq[5], w_tiled=tiled)
+    part_ops = [aq[0][:m_part].clone(), aq[1][:m_part].clone(), aq[2][:m_part].clone()]
+    part_sf = [aq[3 + i][:abi.sf_bytes(m_part, kseg, abi.MG_OPERAND_A)].clone() for i, kseg in enumerate((kn, ks, ko))]
+    part = abi.matmul(part_ops[0], bq[0], part_ops[1], bq[1], part_ops[2], bq[2], part_sf[0], bq[3], part_sf[1], bq[4],
+                      part_sf[2], bq[5], w_tiled=tiled)
+    torch.cuda.synchronize()
+    assert torch.equal(full[:m_part], part)
+    qx, qw = _oracle_operands(x, w, idx, kn, ks, ko)
+    _check_gemm(full, qx, qw, "mixed tile heights")
+
+
 @pytest.mark.parametrize("m", [257, 258, 261, 263, 271, 272, 273, 384, 385, 511, 16, 129, 200])
 @pytest.mark.parametrize("n,kn,ks,ko", [(2048, 2560, 1408, 128), (512, 448, 416, 224)])
 def test_exact_size_activation_buffers_on_the_whole_tile_kernel(abi, m, n, kn, ks, ko):

@@ -1,24 +1,24 @@
 // Mixed block-scaled GEMM for large whole-tile shapes: 256 x 256 workgroup tiles, one workgroup
-// of 4 waves per CU, each wave 128 features x 128 tokens = 4 x 4 tiles of
-// v_mfma_scale_f32_32x32x64_f8f6f4 (256 accumulator registers).  Replaces the three CUTLASS GEMMs
+// of 8 waves per CU (two per SIMD), each wave 128 features x 64 tokens = 4 x 2 tiles of
+// v_mfma_scale_f32_32x32x64_f8f6f4 (128 accumulator registers).  Replaces the three CUTLASS GEMMs
 // of the reference (src/fp4.cu:35, src/fp6.cu:35, src/fp8.cu:35, driver src/gemm.cu:22-47) for
-// M, N multiples of 256 and every K segment at least 128 wide (a multiple of 32).
+// N a multiple of 8 and every K segment at least 128 wide (a multiple of 32), or absent.
 //
-// With one wave per SIMD nothing hides a wave's own instruction issue: next to an MFMA (32 cycles
-// in the matrix pipe) a wave gets only a handful of other instructions for free, so the steady
-// state is written to need about two per MFMA:
-//   * operands and scale atoms go global -> LDS directly (global_load_lds_dwordx4); a copy is a
-//     scalar base (advanced once per stage), a per-lane offset fixed for the segment, and an LDS
+// Next to an MFMA (32 cycles in the matrix pipe) a wave gets only a handful of other instructions
+// for free; with two waves per SIMD one wave's copy and fragment-read instructions issue while the
+// other's MFMA runs (with one wave of 128 x 128 per SIMD the K loop took 10 % more cycles), and the
+// steady state is written to need few of them:
+//   * operands and scale atoms go global -> LDS directly (global_load_lds_dwordx4 / _dword); a copy
+//     is a scalar base (advanced once per stage), a per-lane offset fixed for the segment, and an LDS
 //     offset that is an immediate (the three stage buffers are three copies of the loop body);
 //   * fragment reads use per-lane LDS addresses fixed for the segment plus immediates;
-//   * copies are spread between the MFMAs (the address unit needs about two MFMA times for one
-//     copy of each of the four waves).
+//   * copies are spread between the MFMAs, one after every second MFMA.
 // Pipeline per K stage q (128 elements), three LDS buffers:
-//   read second half of q | 16 MFMAs first half, last copies of q+2 | own reads done, own copies
+//   read second half of q | 8 MFMAs first half, last copies of q+2 | own reads done, own copies
 //   of q+1 landed (those of q+2 stay in flight) | barrier | read first half + scales of q+1 |
-//   16 MFMAs second half, first copies of q+3 into the buffer stage q just freed.
-// The last three stages of a segment copy stages of the next segment(s); they run a generic body
-// whose copy format is a run-time, wave-uniform value.
+//   8 MFMAs second half, first copies of q+3 into the buffer stage q just freed.
+// The last three stages of a segment copy stages of the next segment(s); plans whose segments are
+// too short for that run a generic body whose copy format is a run-time, wave-uniform value.
 // The result tile is transposed through LDS so that stores write 256 contiguous bytes per row.
 #include "mg_common.h"
 
@@ -36,9 +36,18 @@ constexpr int kXOff = 16 * kBlk;          // 16640
 constexpr int kSOff = kXOff + 32 * kBlk;  // E4M3 worst case: two K halves x 16 blocks -> 49920
 constexpr int kStage = kSOff + 2048;      // 51968
 constexpr int kBuffers = 3;
-constexpr int kCopySlots = 13;            // 4 weight copies, up to 8 token copies, 1 scale copy per wave and stage
 constexpr int kStartSkew = 8000;          // see the kernel: largest start delay, in ticks of s_memtime (about 4 us)
-constexpr int kSplit = 5;                 // slots [0, kSplit) go out in the second half of a stage, the rest in the next first half
+
+// Eight waves per workgroup, two per SIMD: a wave's tile is 128 features x 32 * TM tokens (TM = 2: the workgroup's
+// tile is 256 x 256; TM = 1: 256 x 128), 64 * TM accumulator registers, so that two waves fit a SIMD's register file
+// and one wave's copy and fragment-read instructions issue while the other's MFMA runs.  A stage's copies are dealt to
+// the waves so that the workgroup moves every byte exactly once: per wave 2 weight blocks, 2 / 3 / 4 token copies
+// (E2M1 / E3M2 / E4M3) and a quarter of a scale atom pair (a 4-byte copy).
+constexpr int kWaves = 8;
+constexpr int kWCopies = 2;                            // weight copy blocks per wave and stage
+constexpr int kXSlots = 4;                             // token copy slots per wave and stage (E4M3 uses them all)
+constexpr int kCopySlots = kWCopies + kXSlots + 1;     // + the scale copy
+constexpr int kSplit = 3;                              // slots [0, kSplit) go out in the second half of a stage, the rest in the next first half
 
 typedef int v6i __attribute__((ext_vector_type(6)));
 
@@ -98,9 +107,8 @@ template <> struct Fmt<kFmtE4M3> { static constexpr int seg = 2, row_bytes = 128
 // tokens: 16 rows x 64 B (a lane quad reads 64 contiguous bytes of one row), rows j, j+16, ...,
 // j+240 of the tile into block j at j * 1040 (E4M3: one set of 16 blocks per 64-wide K half).
 // E3M2 rows are 96 B: three instructions move the 32 rows j, j+8, ..., j+248 as one row-major
-// block of 3072 B at j * 3088.  Slot 12: waves 0, 2 copy the two weight scale atoms of the stage,
-// waves 1, 3 the two token scale atoms (twice the same bytes to the same place, so that every
-// wave issues the same number of copies and waits with the same count).
+// block of 3072 B at j * 3088.  Last slot: the stage's four scale atoms (two of the features, two
+// of the tokens, 2 KB) as eight 4-byte copies, one per wave.
 // ---------------------------------------------------------------------------------------------
 
 // global[base + voff(lane)] -> LDS[lds_off + 16 * lane]; base and lds_off are wave-uniform
@@ -131,8 +139,24 @@ __device__ __forceinline__ void copy16io(const uint8_t* base, unsigned voff, uns
                : : "v"(voff), "s"(base), "s"(lds_sreg), "n"(OFF - GOFF), "n"(GOFF) : "memory", "m0", "scc");
 }
 
+// 4-byte copies: global[base + voff(lane)] -> LDS[lds_off + 4 * lane] (a quarter of a scale atom pair per wave)
+__device__ __forceinline__ void copy4(const uint8_t* base, unsigned voff, unsigned lds_off) {
+  base = uni(base);
+  lds_off = __builtin_amdgcn_readfirstlane(lds_off);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+               : : "v"(voff), "s"(base), "s"(lds_off) : "memory", "m0");
+}
+template <int OFF>
+__device__ __forceinline__ void copy4i(const uint8_t* base, unsigned voff, unsigned lds_sreg) {
+  base = uni(base);
+  lds_sreg = __builtin_amdgcn_readfirstlane(lds_sreg);
+  asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+               : : "v"(voff), "s"(base), "s"(lds_sreg), "n"(OFF) : "memory", "m0", "scc");
+}
+
 struct Ctx {
   int n0, m0, lane, wave, wn, wm, total;
+  int xatom, xtile;    // the wave's token tiles: scale atom (of 128 rows) of the workgroup's tile, and the first one's index (0 ... 3) in that atom
   int rows_avail;      // activation rows that may be read from m0 on (codes and scales); 1 ... 256
   int cols_avail;      // features of the tile that exist (weight rows and scales that may be read from n0 on); 1 ... 256
   unsigned lds_base;   // LDS byte offset of the dynamic shared memory
@@ -142,7 +166,7 @@ struct Ctx {
 // Token rows are clamped to the last readable row of the tile (rows_avail - 1): in the last, partial
 // token tile the lanes of rows past it copy that row again, into LDS rows of tokens that are never stored.
 struct LaneOffsets {
-  unsigned s0, s1, s2;      // scale atoms: lanes 0-31 the first 128 rows, 32-63 the next 128
+  unsigned s0, s1, s2;      // the wave's quarter of a segment's scale atom pair, 4 bytes per lane
   int lane, wave, last_row, last_col, prow;
 
   __device__ __forceinline__ LaneOffsets(const Plan& p, const Ctx& cx) {
@@ -154,29 +178,30 @@ struct LaneOffsets {
     // fragment end up 512 B apart in their block, which the LDS reads conflict-free (64 B apart they collide)
     const unsigned k = lane >> 2, pr = 2 * (k & 7) + (k >> 3);
     prow = 16 * pr;
-    // scale atoms: waves 0 and 2 copy the feature atoms, 1 and 3 the token atoms; the second atom of a
-    // tile exists only past 128 features / readable token rows
-    const unsigned hi = ((wave & 1) ? cx.rows_avail : cx.cols_avail) <= 128 ? 0 : lane >> 5, lo = (lane & 31) * 16;
+    // scale atoms: waves 0-3 copy a quarter each (256 bytes, 4 per lane) of the tile's two feature atoms, waves 4-7
+    // of its two token atoms; the second atom of a tile exists only past 128 features / readable token rows
+    const unsigned hi = (wave >= 4 ? cx.rows_avail : cx.cols_avail) <= 128 ? 0 : (wave >> 1) & 1;
+    const unsigned lo = (wave & 1) * 256 + lane * 4;
     s0 = hi * ((p.blk0 + 3) >> 2) * 512 + lo;
     s1 = hi * ((p.blk1 + 3) >> 2) * 512 + lo;
     s2 = hi * ((p.blk2 + 3) >> 2) * 512 + lo;
   }
 
   // Byte offset, from the tile's first weight row, that this lane reads in weight copy k of a stage (row-major
-  // weights, row pitch ldb): 64 bytes of row 4 * wave + k + 16 * pr, clamped to the last feature that exists.
+  // weights, row pitch ldb): 64 bytes of row 2 * wave + k + 16 * pr, clamped to the last feature that exists.
   __device__ __forceinline__ unsigned woff(int k, unsigned ldb) const {
-    return (unsigned)min(prow + 4 * wave + k, last_col) * ldb + (lane & 3) * 16;
+    return (unsigned)min(prow + kWCopies * wave + k, last_col) * ldb + (lane & 3) * 16;
   }
 
   // Byte offset, from the tile's first token row, that this lane reads in token copy kx of a stage of
-  // segment sg (row pitch lda).  E2M1: rows 4 * wave + kx + 16 * pr, 16-byte piece lane % 4; E4M3: rows
-  // 8 * (wave % 2) + kx + 16 * pr; E3M2: piece c % 6 of row 2 * wave + kx / 3 + 8 * (c / 6), c = 64 * (kx % 3) + lane.
+  // segment sg (row pitch lda).  E2M1: rows 2 * wave + kx + 16 * pr, 16-byte piece lane % 4; E4M3: rows
+  // 4 * (wave % 4) + kx + 16 * pr; E3M2: piece c % 6 of row wave + 8 * (c / 6), c = 64 * kx + lane.
   __device__ __forceinline__ unsigned xoff(int sg, int kx, unsigned lda) const {
     if (sg == 1) {
-      const int c = 64 * (kx % 3) + lane;
-      return (unsigned)min(8 * (c / 6) + 2 * wave + kx / 3, last_row) * lda + (c % 6) * 16;
+      const int c = 64 * kx + lane;
+      return (unsigned)min(8 * (c / 6) + wave, last_row) * lda + (c % 6) * 16;
     }
-    const int first = sg == 0 ? 4 * wave : 8 * (wave & 1);
+    const int first = sg == 0 ? 2 * wave : 4 * (wave & 3);
     return (unsigned)min(prow + first + kx, last_row) * lda + (lane & 3) * 16;
   }
 };
@@ -206,14 +231,14 @@ struct StageBases {
     if (plan.w_tiled) {
       // 16 KB per (feature tile, stage), 1 KB per copy block: the wave's 4 blocks are consecutive
       const unsigned nstg = (unsigned)pick3(sg, (uint64_t)plan.st0, (uint64_t)plan.st1, (uint64_t)plan.st2);
-      w = pb + (((size_t)(c.n0 >> 8) * nstg + ql) * 16 + c.wave * 4) * 1024;
+      w = pb + (((size_t)(c.n0 >> 8) * nstg + ql) * 16 + c.wave * kWCopies) * 1024;
       ldb = 1024;
     } else {
       w = pb + (size_t)c.n0 * ldb + (size_t)ql * 64;   // the lanes' offsets carry the wave's rows
     }
-    // the tile's first token row (the lanes' offsets carry the wave's rows); E4M3: K half wave / 2
-    x = pa + (size_t)c.m0 * lda + (size_t)ql * rb + (sg == 2 ? (c.wave >> 1) * 64 : 0);
-    s = (c.wave & 1) == 0 ? psb + ((size_t)(c.n0 >> 7) * nst + ql) * 512 : psa + ((size_t)(c.m0 >> 7) * nst + ql) * 512;
+    // the tile's first token row (the lanes' offsets carry the wave's rows); E4M3: K half wave / 4
+    x = pa + (size_t)c.m0 * lda + (size_t)ql * rb + (sg == 2 ? (c.wave >> 2) * 64 : 0);
+    s = c.wave < 4 ? psb + ((size_t)(c.n0 >> 7) * nst + ql) * 512 : psa + ((size_t)(c.m0 >> 7) * nst + ql) * 512;
   }
 };
 
@@ -227,27 +252,26 @@ struct GenericCopy {
       : b(plan, q, c), buf(c.lds_base + (q % kBuffers) * kStage) {}
 
   __device__ __forceinline__ int count() const {
-    return b.seg < 0 ? 0 : 4 + (b.seg == 0 ? 4 : (b.seg == 1 ? 6 : 8)) + 1;
+    return b.seg < 0 ? 0 : kWCopies + (b.seg == 0 ? kXSlots / 2 : (b.seg == 1 ? 3 * kXSlots / 4 : kXSlots)) + 1;
   }
 
   template <int K>
   __device__ __forceinline__ void issue(const LaneOffsets& lo, int wave) const {
     if (b.seg < 0) return;
-    if constexpr (K < 4) {
-      if (b.tiled) copy16(b.w + (size_t)K * 1024, lo.lane * 16, buf + kWOff + (wave * 4 + K) * kBlk);
-      else copy16(b.w, lo.woff(K, b.ldb), buf + kWOff + (wave * 4 + K) * kBlk);
-    } else if constexpr (K < 12) {
-      constexpr int kx = K - 4;
+    if constexpr (K < kWCopies) {
+      if (b.tiled) copy16(b.w + (size_t)K * 1024, lo.lane * 16, buf + kWOff + (wave * kWCopies + K) * kBlk);
+      else copy16(b.w, lo.woff(K, b.ldb), buf + kWOff + (wave * kWCopies + K) * kBlk);
+    } else if constexpr (K < kCopySlots - 1) {
+      constexpr int kx = K - kWCopies;
       if (b.seg == 0) {
-        if constexpr (kx < 4) copy16(b.x, lo.xoff(0, kx, b.lda), buf + kXOff + (wave * 4 + kx) * kBlk);
+        if constexpr (kx < kXSlots / 2) copy16(b.x, lo.xoff(0, kx, b.lda), buf + kXOff + (wave * (kXSlots / 2) + kx) * kBlk);
       } else if (b.seg == 1) {
-        if constexpr (kx < 6)
-          copy16(b.x, lo.xoff(1, kx, b.lda), buf + kXOff + (wave * 2 + kx / 3) * kBlk6 + (kx % 3) * 1024);
+        if constexpr (kx < 3 * kXSlots / 4) copy16(b.x, lo.xoff(1, kx, b.lda), buf + kXOff + wave * kBlk6 + kx * 1024);
       } else {
-        copy16(b.x, lo.xoff(2, kx, b.lda), buf + kXOff + (wave * 8 + kx) * kBlk);
+        copy16(b.x, lo.xoff(2, kx, b.lda), buf + kXOff + (wave * kXSlots + kx) * kBlk);
       }
     } else {
-      copy16(b.s, pick3u(b.seg, lo.s0, lo.s1, lo.s2), buf + kSOff + (wave & 1) * 1024);
+      copy4(b.s, pick3u(b.seg, lo.s0, lo.s1, lo.s2), buf + kSOff + wave * 256);
     }
   }
 };
@@ -266,16 +290,16 @@ __device__ __forceinline__ void issue_range(const GenericCopy& cp, const LaneOff
 // weight copies; vw[] is then unused.
 template <int FMT, bool WT>
 struct LeanCopy {
-  static constexpr int NX = Fmt<FMT>::x_copies;
-  // token copies, rows clamped to the last readable one.  E2M1: one offset per copy.  E3M2: one per third
-  // of a block for its first row; bits 0-2 of vs say whether the second row is a row further on.  E4M3,
-  // of which there are few stages: the first copy's offset, and in its bits 0-2 how many of the seven
-  // row steps that follow stay inside the readable rows.  (All offsets are multiples of 16.)
-  static constexpr int NV = FMT == kFmtE4M3 ? 1 : (FMT == kFmtE3M2 ? 3 : 4);
+  static constexpr int WC = kWCopies;
+  static constexpr int NX = Fmt<FMT>::x_copies / 2;
+  // token copies, rows clamped to the last readable one.  E2M1, E3M2: one offset per copy.  E4M3, of which
+  // there are few stages: the first copy's offset, and in its bits 0-2 how many of the three row steps that
+  // follow stay inside the readable rows.  (These offsets are multiples of 16.)
+  static constexpr int NV = FMT == kFmtE4M3 ? 1 : (FMT == kFmtE3M2 ? 3 : NX);
   const uint8_t *w, *x, *s;        // bases of the stage being copied
   unsigned lds_w, lds_x, lds_s;    // LDS offsets of the wave's first weight / token block and scale atom pair in buffer 0
   unsigned lda;
-  unsigned vw[4], vx[NV], vs, vlin;
+  unsigned vw[WC], vx[NV], vs, vlin;
 
   __device__ __forceinline__ void init(const Plan& plan, int q, const LaneOffsets&, const Ctx& c) {
     const LaneOffsets lo(plan, c);   // recomputed here rather than kept in registers across the K loop
@@ -287,28 +311,24 @@ struct LeanCopy {
     vlin = c.lane * 16;
     if constexpr (!WT) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) vw[k] = lo.woff(k, b.ldb);
+      for (int k = 0; k < WC; ++k) vw[k] = lo.woff(k, b.ldb);
     }
     lda = __builtin_amdgcn_readfirstlane(b.lda);
-    unsigned flags = 0;
     if constexpr (FMT == kFmtE4M3) {
-      const int row0 = lo.prow + 8 * (c.wave & 1);
-      vx[0] = lo.xoff(2, 0, b.lda) | (unsigned)min(max(lo.last_row - row0, 0), 7);
+      const int row0 = lo.prow + 4 * (c.wave & 3);
+      vx[0] = lo.xoff(2, 0, b.lda) | (unsigned)min(max(lo.last_row - row0, 0), NX - 1);
     } else if constexpr (FMT == kFmtE3M2) {
 #pragma unroll
-      for (int t = 0; t < 3; ++t) {
-        vx[t] = lo.xoff(1, t, b.lda);
-        flags |= (lo.xoff(1, 3 + t, b.lda) != vx[t] ? 1u : 0u) << t;
-      }
+      for (int t = 0; t < 3; ++t) vx[t] = lo.xoff(1, t, b.lda);
     } else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) vx[k] = lo.xoff(0, k, b.lda);
+      for (int k = 0; k < NX; ++k) vx[k] = lo.xoff(0, k, b.lda);
     }
-    vs = (sg == 0 ? lo.s0 : (sg == 1 ? lo.s1 : lo.s2)) | flags;
-    lds_w = __builtin_amdgcn_readfirstlane(c.lds_base + kWOff + c.wave * 4 * kBlk);
+    vs = sg == 0 ? lo.s0 : (sg == 1 ? lo.s1 : lo.s2);
+    lds_w = __builtin_amdgcn_readfirstlane(c.lds_base + kWOff + c.wave * WC * kBlk);
     lds_x = __builtin_amdgcn_readfirstlane(c.lds_base + kXOff +
-                                           c.wave * (FMT == kFmtE2M1 ? 4 * kBlk : (FMT == kFmtE3M2 ? 2 * kBlk6 : 8 * kBlk)));
-    lds_s = __builtin_amdgcn_readfirstlane(c.lds_base + kSOff + (c.wave & 1) * 1024);
+                                           c.wave * (FMT == kFmtE3M2 ? kBlk6 : NX * kBlk));
+    lds_s = __builtin_amdgcn_readfirstlane(c.lds_base + kSOff + c.wave * 256);
   }
 
   __device__ __forceinline__ void advance() {
@@ -317,24 +337,22 @@ struct LeanCopy {
     s += 512;
   }
 
-  static constexpr int count() { return 4 + NX + 1; }
+  static constexpr int count() { return WC + NX + 1; }
 
   // slot K into the stage buffer at byte offset boff (wave-uniform)
   template <int K>
   __device__ __forceinline__ void issue(unsigned boff) const {
-    if constexpr (K < 4) {
+    if constexpr (K < WC) {
       if constexpr (WT) copy16io<K * kBlk, K * 1024>(w, vlin, lds_w + boff);
       else copy16i<K * kBlk>(w, vw[K], lds_w + boff);
-    } else if constexpr (K < 4 + NX) {
-      constexpr int kx = K - 4;
-      if constexpr (FMT == kFmtE3M2)
-        copy16i<(kx / 3) * kBlk6 + (kx % 3) * 1024>(x, kx < 3 ? vx[kx] : vx[kx - 3] + ((vs >> (kx - 3)) & 1) * lda,
-                                                    lds_x + boff);
+    } else if constexpr (K < WC + NX) {
+      constexpr int kx = K - WC;
+      if constexpr (FMT == kFmtE3M2) copy16i<kx * 1024>(x, vx[kx], lds_x + boff);
       else if constexpr (FMT == kFmtE4M3)
         copy16i<kx * kBlk>(x, (vx[0] & ~15u) + min((unsigned)kx, vx[0] & 7u) * lda, lds_x + boff);
       else copy16i<kx * kBlk>(x, vx[kx], lds_x + boff);
-    } else if constexpr (K == 12) {
-      copy16i<0>(s, FMT == kFmtE3M2 ? vs & ~15u : vs, lds_s + boff);
+    } else if constexpr (K == kCopySlots - 1) {
+      copy4i<0>(s, vs, lds_s + boff);
     }
   }
 };
@@ -398,12 +416,12 @@ struct WeightPtrs {
   const uint8_t* sw;   // scale dwords of the 4 feature tiles
   const uint8_t* sx;   // scale dwords of the 4 token tiles
 
-  // tm: token tiles of 32 per wave (4: a wave's tokens are one scale atom of 128 rows; 2: both halves share one)
-  __device__ __forceinline__ WeightPtrs(const uint8_t* lds, const Ctx& c, int tm) {
+  // the wave's token tiles lie in scale atom c.xatom of the workgroup's tile
+  __device__ __forceinline__ WeightPtrs(const uint8_t* lds, const Ctx& c) {
     const int i = c.lane & 31, g = c.lane >> 5;
     w = lds + kWOff + (i & 15) * kBlk + (i >> 4) * 512 + c.wn * 256 + g * 16;
     sw = lds + kSOff + c.wn * 512 + i * 16;
-    sx = lds + kSOff + 1024 + (tm == 4 ? c.wm * 512 : 0) + i * 16;
+    sx = lds + kSOff + 1024 + c.xatom * 512 + i * 16;
   }
 };
 
@@ -479,15 +497,17 @@ struct Scales {
   int w[4], x[TM];   // scale dwords of the 4 feature / TM token tiles, shifted so that byte 0 / 2 is block g / 2+g
 };
 
-// sx holds the dwords of the four token tiles of a scale atom; with TM == 2 the wave's are 2 * wm and 2 * wm + 1
+// sx holds the dwords of the four token tiles of a scale atom; the wave's are xtile ... xtile + TM - 1 (xtile wave-uniform)
 template <int TM>
-__device__ __forceinline__ void shift_scales(Scales<TM>& sc, v4i sw, v4i sx, int lane, int wm) {
+__device__ __forceinline__ void shift_scales(Scales<TM>& sc, v4i sw, v4i sx, int lane, int xtile) {
   const int g8 = (lane >> 5) * 8;
 #pragma unroll
   for (int t = 0; t < 4; ++t) sc.w[t] = (int)((unsigned)sw[t] >> g8);
 #pragma unroll
   for (int t = 0; t < TM; ++t) {
-    const int v = TM == 4 ? sx[t] : (wm ? sx[2 + t] : sx[t]);
+    int v;
+    if constexpr (TM == 2) v = xtile ? sx[2 + t] : sx[t];
+    else v = xtile == 0 ? sx[0] : (xtile == 1 ? sx[1] : (xtile == 2 ? sx[2] : sx[3]));
     sc.x[t] = (int)((unsigned)v >> g8);
   }
 }
@@ -500,13 +520,16 @@ __device__ __forceinline__ void mfma_one(v16f& acc, v4i w, const typename Fmt<FM
   acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(widen(w), widen(x), acc, kFmtE2M1, FMT, 2 * H, scw, 2 * H, scx);
 }
 
-// first copy slot >= K that a stage of format FMT has (slots 4 + x_copies .. 11 are empty)
+// first copy slot >= K that a stage of format FMT has (the token slots past the format's copies are empty)
 template <int FMT>
-constexpr int next_slot(int k) { return (k >= 4 + Fmt<FMT>::x_copies && k < 12) ? 12 : k; }
+constexpr int next_slot(int k) {
+  return (k >= kWCopies + Fmt<FMT>::x_copies / 2 && k < kCopySlots - 1) ? kCopySlots - 1 : k;
+}
 
-// 16 MFMAs of one K half.  Between them: the fragment reads of `rd` (for the next half: one after
-// each of the first MFMAs, so that the four waves do not all queue at the LDS at once with their
-// MFMAs stuck behind) and the copy slots [K0, K1) of one stage, one after every second MFMA.
+// The 4 * TM MFMAs of one K half.  Between them: the fragment reads of `rd` (for the next half: one after
+// each of the first MFMAs -- two where a half has fewer MFMAs than reads --, so that the waves do not all
+// queue at the LDS at once with their MFMAs stuck behind) and the copy slots [K0, K1) of one stage, one after
+// every second MFMA of 8, after every one of 4.
 // LEAN: slots of `lc` (a stage of format CF, skipped when !on) into the buffer at byte offset boff;
 // otherwise slots of the run-time plan `gc`.
 template <int FMT, int H, bool LEAN, int CF, int M0, int K0, int K1, class Reader, bool WT, int TM>
@@ -516,10 +539,15 @@ __device__ __forceinline__ void mfma_half(v16f (&acc)[4][TM], const HalfFrags<FM
   if constexpr (M0 < 4 * TM) {
     constexpr int tn = M0 / TM, tm = M0 % TM;
     mfma_one<FMT, H>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
-    if constexpr (M0 < Reader::kReads) rd.template read<M0>();
+    // one fragment read per MFMA, two where a half has fewer MFMAs than reads (TM == 1)
+    constexpr int RP = (Reader::kReads + 4 * TM - 1) / (4 * TM);
+    if constexpr (M0 * RP < Reader::kReads) rd.template read<M0 * RP>();
+    if constexpr (RP == 2 && M0 * RP + 1 < Reader::kReads) rd.template read<M0 * RP + 1>();
+    static_assert(RP <= 2, "fragment reads per MFMA");
     constexpr int KS = LEAN ? (CF == kFmtNone ? K1 : next_slot<CF>(K0)) : K0;
-    // a copy slot after every second MFMA of 16, after every one of 8
-    if constexpr ((TM == 2 || (M0 & 1) == 1) && KS < K1) {
+    // a copy slot after every second MFMA where a wave has twice as many MFMAs per half as copy slots, else after every one
+    constexpr bool kEvery = 4 * TM <= kCopySlots - kSplit;
+    if constexpr ((kEvery || (M0 & 1) == 1) && KS < K1) {
       if constexpr (LEAN) {
         if (on) lc.template issue<KS>(boff);
       } else {
@@ -591,7 +619,7 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][TM], HalfFrags<FMT, TM
   mfma_half<FMT, 1, LEAN, CE, 0, 0, kSplit>(acc, b, sc, rd_n, lce, early_on, ring.cur, gc, lo, c.wave);
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
-  shift_scales(sc, sw, sx, c.lane, c.wm);
+  shift_scales(sc, sw, sx, c.lane, c.xtile);
   if constexpr (FR == FMT) a = nx;
   else a_next = nx;
 }
@@ -843,22 +871,25 @@ __device__ __forceinline__ Plan start_workgroup(const Plan& plan_arg, int first_
 // REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
 // SEGS: which activation segments the plan has, bit 0 E2M1 (always), bit 1 E3M2, bit 2 E4M3 -- the
 // prefetched fragments pass from a segment to the next one that exists, and their types are fixed here.
-// TM: token tiles of 32 per wave.  4: the workgroup's tile is 256 features x 256 tokens.  2: 256 x 128, for
+// TM: token tiles of 32 per wave.  2: the workgroup's tile is 256 features x 256 tokens.  1: 256 x 128, for
 // problems with fewer than 256 whole tiles (every CU still gets a workgroup): same copies (the lanes of token
 // rows 128 ... 255 read the last row again, which costs the address unit next to nothing), same LDS image,
 // half the MFMAs per stage, a copy slot after every MFMA instead of every second one.
 // NLAST: see run_segment (the launcher picks the instance from the plan).
-// Computes one tile of 256 features x 64 * TM tokens: feature tile tile_n, token tile tile_m (of 64 * TM rows).
+// Computes one tile of 256 features x 128 * TM tokens: feature tile tile_n, token tile tile_m (of 128 * TM rows).
 template <bool REGULAR, bool REM, bool WT, int SEGS, int TM, int NLAST>
 __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int tile_m, int tiles_n, int N, int m_store,
                                              int a_rows, uint16_t* __restrict__ d, uint8_t* lds) {
+  static_assert(TM == 2 || TM == 1, "wave tiles of 128 features x 32 * TM tokens");
   const int tid = threadIdx.x;
   Ctx c;
   c.lane = tid & 63;
   c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   c.wn = c.wave & 1;
   c.wm = c.wave >> 1;
-  constexpr int kTokens = 64 * TM;   // token rows of the workgroup's tile
+  c.xatom = (c.wm * TM) >> 2;
+  c.xtile = (c.wm * TM) & 3;
+  constexpr int kTokens = 16 * kWaves * TM;   // token rows of the workgroup's tile
   c.n0 = tile_n * kT;
   c.m0 = tile_m * kTokens;
   c.total = plan.total;
@@ -867,7 +898,7 @@ __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int t
   c.lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t*)lds;
 
   const LaneOffsets lo(plan, c);
-  const WeightPtrs wp(lds, c, TM);
+  const WeightPtrs wp(lds, c);
 
   // the blocks past the whole stages first (see RemainderHalf): first K halves requested ahead of the copies
   RemainderHalf<kFmtE2M1, TM> p0;
@@ -960,7 +991,7 @@ __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int t
     const FragReader<kFmtE2M1, 0, true, TM> rd{a4, sw, sx, wp.w, xp.x, wp.sw, wp.sx, true};
     read_all(rd);
     wait_lds_reads();
-    shift_scales(sc, sw, sx, c.lane, c.wm);
+    shift_scales(sc, sw, sx, c.lane, c.xtile);
   }
   LeanCopy<kFmtNone, WT> l0;
   if constexpr (SEGS == 7) {
@@ -983,7 +1014,7 @@ __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int t
   // No barrier: the last stage reads no fragments after its barrier, before which every wave's copies had landed,
   // and from here on a wave touches only its own part of the LDS.
   constexpr int kPitch = 256 + 16;   // bytes per token row in LDS
-  static_assert(4 * 128 * kPitch <= kBuffers * kStage, "epilogue staging must fit the stage buffers");
+  static_assert(kWaves * 32 * TM * kPitch <= kBuffers * kStage, "epilogue staging must fit the stage buffers");
   uint8_t* stage = lds + c.wave * (32 * TM) * kPitch;
   {
     const int g = c.lane >> 5;
@@ -1030,8 +1061,8 @@ __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int t
 }
 
 
-template <bool REGULAR, bool REM, bool WT, int SEGS = 7, int TM = 4, int NLAST = 0>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+template <bool REGULAR, bool REM, bool WT, int SEGS = 7, int TM = 2, int NLAST = 0>
+__global__ void __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
 mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d, int first_round,
                       int skew) {
   extern __shared__ __align__(16) uint8_t lds[];
@@ -1043,10 +1074,11 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
 
 // The same for problems whose last round of 256 x 256 tiles would leave at least half of the CUs idle: the first
 // n_whole workgroups compute whole tiles (n_whole a multiple of the CU count), the others the remaining whole tiles
-// as two tiles of 256 x 128 each.  A half tile takes about 0.7 of a whole tile's time, and the half-empty round took
-// as long as a full one (M = 3072 and 4096 at N = 14336, K = 4096: 768 tiles 101.5 us, 896 tiles 134.1 us).
+// as two tiles of 256 x 128 each.  Measured: M = 4096, N = 5120, K = 8576 / 4800 / 448 (320 tiles) 166 -> 147 us; where the
+// last round is exactly half full (M = 4096, N = 14336: 896 tiles) it changes nothing -- the chip is at its power limit,
+// and the CUs that work while the others idle get the clock the others do not use.
 template <bool REM, bool WT, int NLAST>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ void __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
 mixed_gemm_256_tail_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows, uint16_t* __restrict__ d, int first_round,
                            int skew, int n_whole) {
   extern __shared__ __align__(16) uint8_t lds[];
@@ -1056,13 +1088,13 @@ mixed_gemm_256_tail_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a
   int tile_n, tile_m;
   if (wg < n_whole) {
     tile_of(wg, ntiles, tiles_n, tile_n, tile_m);
-    compute_tile<true, REM, WT, 7, 4, NLAST>(plan, tile_n, tile_m, tiles_n, N, m_store, a_rows, d, lds);
+    compute_tile<true, REM, WT, 7, 2, NLAST>(plan, tile_n, tile_m, tiles_n, N, m_store, a_rows, d, lds);
   } else {
     const int h = wg - n_whole;
     tile_of(n_whole + (h >> 1), ntiles, tiles_n, tile_n, tile_m);
     const int half_m = 2 * tile_m + (h & 1);
     if (half_m * 128 >= m_store) return;   // the lower half of a ragged last tile: no token of it exists
-    compute_tile<true, REM, WT, 7, 2, NLAST>(plan, tile_n, half_m, tiles_n, N, m_store, a_rows, d, lds);
+    compute_tile<true, REM, WT, 7, 1, NLAST>(plan, tile_n, half_m, tiles_n, N, m_store, a_rows, d, lds);
   }
 }
 
@@ -1086,9 +1118,8 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
 }
 
 // Token rows per workgroup tile for a problem of m_store tokens: 256, or 128 when the 256 x 256 tiles would leave
-// at least half of the CUs without one.  A half tile takes about 0.8 of a whole tile's time (the copies of a stage
-// bound it, not its MFMAs), so halves pay only where they put idle CUs to work: measured, M = 2048 N = 4096
-// K = 14336 (128 whole tiles) 99 -> 84 us, M = 1024 N = 4096 K = 4096 (64) 28 -> 22 us, but 896 whole tiles 145 -> 170 us.
+// at least half of the CUs without one.  A half tile takes most of a whole tile's time (the copies of a stage
+// bound it, not its MFMAs), so halves pay only where they put idle CUs to work.
 static int tile_tokens(int m_store, int N, int cus) {
   const long long tiles = (long long)((m_store + kT - 1) / kT) * ((N + kT - 1) / kT);
   return tiles <= cus / 2 ? 128 : 256;
@@ -1144,13 +1175,14 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   const int segs = 1 | (KS > 0 ? 2 : 0) | (KO > 0 ? 4 : 0);
   const int last_stages = KO > 0 ? KO / 128 : (KS > 0 ? KS / 128 : KN / 128);
   const int nlast = last_stages >= 3 ? 3 : last_stages;
+  // token tiles of 32 per wave: 2 for 256 x 256 workgroup tiles, 1 for 256 x 128
   kernel_t kernel = nullptr;
   if (rem) {
-    if (w_tiled) kernel = half ? select_kernel<true, true, 2>(regular, segs, nlast) : select_kernel<true, true, 4>(regular, segs, nlast);
-    else kernel = half ? select_kernel<true, false, 2>(regular, segs, nlast) : select_kernel<true, false, 4>(regular, segs, nlast);
+    if (w_tiled) kernel = half ? select_kernel<true, true, 1>(regular, segs, nlast) : select_kernel<true, true, 2>(regular, segs, nlast);
+    else kernel = half ? select_kernel<true, false, 1>(regular, segs, nlast) : select_kernel<true, false, 2>(regular, segs, nlast);
   } else {
-    if (w_tiled) kernel = half ? select_kernel<false, true, 2>(regular, segs, nlast) : select_kernel<false, true, 4>(regular, segs, nlast);
-    else kernel = half ? select_kernel<false, false, 2>(regular, segs, nlast) : select_kernel<false, false, 4>(regular, segs, nlast);
+    if (w_tiled) kernel = half ? select_kernel<false, true, 1>(regular, segs, nlast) : select_kernel<false, true, 2>(regular, segs, nlast);
+    else kernel = half ? select_kernel<false, false, 1>(regular, segs, nlast) : select_kernel<false, false, 2>(regular, segs, nlast);
   }
   if (kernel == nullptr) return hipErrorInvalidValue;
   // a last round of whole tiles on at most half of the CUs: those tiles as twice as many half tiles
@@ -1179,10 +1211,10 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   const int ntiles = tiles_n * tiles_m;
   const int skew = ntiles > lim.cus ? kStartSkew : 0;
   if (tail)
-    hipLaunchKernelGGL(tail_kernel, dim3(ntiles + rest), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,
+    hipLaunchKernelGGL(tail_kernel, dim3(ntiles + rest), dim3(64 * kWaves), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,
                        static_cast<uint16_t*>(d), lim.cus, skew, ntiles - rest);
   else
-    hipLaunchKernelGGL(kernel, dim3(ntiles), dim3(256), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,
+    hipLaunchKernelGGL(kernel, dim3(ntiles), dim3(64 * kWaves), kBuffers * kStage, stream, p, tiles_n, N, m_store, a_rows,
                        static_cast<uint16_t*>(d), lim.cus, skew);
   return hipGetLastError();
 }

@@ -42,6 +42,8 @@ MEASURED_TRAFFIC = {
                  "source": "mixedgemm_amd/csrc/reorder_quant.hip", "sha": "1d89b7fe0d03a81d"},
     "decode_c2": {"bytes": int((16318.0 * 1.99980 + 896.0 * 1.0) * 1024),        # 34.3 MB against 31.4 MB algorithmic (tile-major weights)
                   "source": "mixedgemm_amd/csrc/mixed_gemm.hip", "sha": "a6cdb0f27150abfe"},
+    "quant_w_c3": {"bytes": 0, "source": "mixedgemm_amd/csrc/reorder_quant.hip", "sha": "not profiled yet"},
+    "tile_w_c3": {"bytes": 0, "source": "mixedgemm_amd/csrc/mixed_gemm_256.hip", "sha": "not profiled yet"},
     "calibrate_c1": {"bytes": int(((16411.0 + 1045.0 + 81.5) * 1.99980 + (2048.0 + 16.0 + 56.2) * 1.0) * 1024),   # three kernels
                      "source": "mixedgemm_amd/csrc/calibrate.hip", "sha": "84a260f8dfd73ec0"},
 }
@@ -95,6 +97,11 @@ def quant_bytes(m, k, kn, ks, ko):
 def gemm_bytes(m, n, kn, ks, ko):
     k = kn + ks + ko
     return n * k // 2 + n * k // 32 + m * (kn // 2 + 3 * ks // 4 + ko) + m * k // 32 + m * n * 2
+
+
+def weight_quant_bytes(n, k):
+    """Algorithmic bytes of one weight reorder-quantize launch: bf16 rows in, E2M1 codes and E8M0 scales out, the index once."""
+    return n * (2 * k + k // 2 + k // 32) + 2 * k
 
 
 def event_ms(pairs):
@@ -329,6 +336,44 @@ def main():
             "zero_ms": round(z_ms, 5), "zero_tflops": round(flops / (z_ms * 1e-3) / 1e12, 1),
             "bench_operands_ms": round(r_ms, 5), "bench_operands_tflops": round(flops / (r_ms * 1e-3) / 1e12, 1)}
         del zq, zw, zb
+        # ------------------------------------------------------------ the weight side of the reorder-quantize kernel
+        # (run_reorder_bf16_fp4, timed by bench_reorder.cu:143-166 of the reference next to the activation side):
+        # c3's W[14336, 4096] -> three E2M1 segments + scales, then the tile-major rewrite of the codes; offline work
+        # in deployment, so outside the headline's step.  Three rotating W (352 MB) and five rotating code sets
+        # (5 x 2 x 29.4 MB) keep the bytes out of the 256 MB Infinity Cache.
+        wsets = [wd] + [H.make_weights(n, k, 2300 + i).to(dev) for i in range(2)]
+        wouts = [abi.alloc_quant_outputs(n, kn, ks, ko, abi.MG_OPERAND_B, dev) for _ in range(3)]
+        for i in range(3):
+            abi.reorder_quantize_w(wsets[i], idd, kn, ks, ko, out=wouts[i])
+        torch.cuda.synchronize()
+        wq_ms = graph_ms(lambda i: abi.reorder_quantize_w(wsets[i % 3], idd, kn, ks, ko, out=wouts[i % 3]), 12)
+        wqb = weight_quant_bytes(n, k)
+        extra["reorder_quant_w_c3"] = {
+            "workload": "weight reorder-quantize of c3's W[14336, 4096] (all E2M1, segments 2560/1408/128), 3 rotating inputs, "
+                        "12 launches replayed as a HIP graph",
+            "value": round(wqb / (wq_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "avg_kernel_ms": round(wq_ms, 5),
+            "roofline": {"bound": "hbm", "achieved": round(wqb / (wq_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(wqb / (wq_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": traffic("quant_w_c3")[0],
+                         "traffic_source": traffic("quant_w_c3")[1], "algorithmic_bytes": wqb}}
+        del wsets
+        csets = [tuple(t.clone() for t in bq[:3]) for _ in range(5)]
+        tsets = [tuple(torch.empty_like(t) for t in bq[:3]) for _ in range(5)]
+
+        def tile(i):
+            for src, dst in zip(csets[i % 5], tsets[i % 5]):
+                abi.check(L.mg_tile_weights(vp(src), vp(dst), src.shape[0], src.shape[1] * 2,
+                                            ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)), "mg_tile_weights")
+
+        tw_ms = graph_ms(tile, 20)
+        twb = 2 * sum(t.numel() for t in bq[:3])
+        extra["tile_weights_c3"] = {
+            "workload": "tile-major rewrite of c3's weight codes (three launches, one per segment: 29.4 MB read + 29.4 MB written), "
+                        "5 rotating sets, 20 calls replayed as a HIP graph",
+            "value": round(twb / (tw_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "avg_ms": round(tw_ms, 5),
+            "roofline": {"bound": "hbm", "achieved": round(twb / (tw_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(twb / (tw_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": traffic("tile_w_c3")[0],
+                         "traffic_source": traffic("tile_w_c3")[1], "algorithmic_bytes": twb}}
+        del csets, tsets, wouts
         # ------------------------------------------------------------ c1: reorder-quantize alone, HBM-bound
         m1, _, k1, kn1, ks1, ko1 = H.CONFIGS["c1"]
         nsets = 8                                    # 8 x 44 MB > 256 MB Infinity Cache
@@ -473,21 +518,23 @@ def main():
                                          "Infinity Cache); 20 launches per kernel replayed as a HIP graph: 0.15 s of untimed replays, then the median of 5", "rows": matrix}
 
         # ------------------------------------------------------------ one activation format at a time (c3's M, N, K)
-        # the 256x256 kernel needs all three segments, so the other two get one 128-wide stage each
+        # splits that run the kernels c3 runs (segment-boundary copies compiled in: at least three stages in each of
+        # the first two segments), tile-major weights; the other two formats get the fewest stages that allows
         per_format = []
-        for name, (knf, ksf, kof) in (("e2m1", (3840, 128, 128)), ("e3m2", (128, 3840, 128)), ("e4m3", (128, 128, 3840))):
+        for name, (knf, ksf, kof) in (("e2m1", (3584, 384, 128)), ("e3m2", (384, 3584, 128)), ("e4m3", (384, 384, 3328))):
             aqf = abi.reorder_quantize_x(xd, idd, knf, ksf, kof)
             wqf = abi.reorder_quantize_w(wd, idd, knf, ksf, kof)
+            wqf = abi.tile_weights(*wqf[:3]) + wqf[3:]
             df = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
             f_ms = graph_ms(lambda i: abi.matmul(aqf[0], wqf[0], aqf[1], wqf[1], aqf[2], wqf[2], aqf[3], wqf[3],
-                                                 aqf[4], wqf[4], aqf[5], wqf[5], out=df), 20)
+                                                 aqf[4], wqf[4], aqf[5], wqf[5], out=df, w_tiled=True), 20)
             pk = blended_peak(knf, ksf, kof)
             tf = 2.0 * m * n * k / (f_ms * 1e-3) / 1e12
             per_format.append({"activations": name, "split": [knf, ksf, kof], "gemm_ms": round(f_ms, 5),
                                "tflops": round(tf, 1), "peak": round(pk, 1), "frac": round(tf / pk, 4)})
             del aqf, wqf, df
-        extra["per_format_gemm"] = {"note": "c3's M, N and K with 3840 of the 4096 channels in one activation format; "
-                                            "peak = the same blended nominal formula", "rows": per_format}
+        extra["per_format_gemm"] = {"note": "c3's M, N and K with 3584 (E4M3: 3328) of the 4096 channels in one activation format, "
+                                            "on the kernels c3 runs; peak = the same blended nominal formula", "rows": per_format}
 
         # ------------------------------------------------------------ plans without E3M2 and / or E4M3 activations
         partial = []

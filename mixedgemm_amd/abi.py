@@ -363,7 +363,8 @@ def calibrate_reorder_index(x, out=None, workspace=None):
     """Reorder index of a bf16 activation sample x[M, K]: channels by ascending max |x| over the
     rows, ties by channel number, int16 (main.py:31-33 of the reference, there as torch calls)."""
     _require(x, torch.bfloat16, "x")
-    assert x.dim() == 2
+    if x.dim() != 2:
+        raise MixedGemmError(f"x: expected a 2-D tensor [rows, channels], got {x.dim()} dimensions")
     m, k = x.shape
     need = int(lib().mg_calibrate_workspace_bytes(k))
     if workspace is None:

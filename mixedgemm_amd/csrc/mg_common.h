@@ -4,6 +4,7 @@
 #include <stdint.h>
 
 #include <mutex>
+#include <unordered_map>
 
 namespace mg {
 
@@ -36,27 +37,21 @@ __host__ __device__ inline size_t sf_offset(int r, int kb, int katoms) {
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // Raises a kernel's dynamic-LDS limit to `bytes`, once per kernel and device (the attribute is kept
-// per device); safe to call from several host threads.
+// per device); safe to call from several host threads.  The library instantiates a few hundred kernels
+// that need it: the record of what has been set is a hash map, so that a process that has launched many of
+// them still pays one look-up per launch and no driver call.
 inline hipError_t allow_dynamic_lds(const void* kernel, int bytes) {
-  struct Entry { const void* kernel; uint64_t devices; };
   static std::mutex mu;
-  static Entry table[32] = {};
+  static std::unordered_map<const void*, uint64_t> done;   // kernel -> bit per device on which the attribute is set
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   const uint64_t bit = 1ull << (dev & 63);
   std::lock_guard<std::mutex> lock(mu);
-  Entry* slot = nullptr;
-  for (Entry& t : table) {
-    if (t.kernel == kernel) { slot = &t; break; }
-    if (t.kernel == nullptr && slot == nullptr) slot = &t;
-  }
-  if (slot != nullptr && slot->kernel == kernel && (slot->devices & bit)) return hipSuccess;
+  uint64_t& devices = done[kernel];
+  if (devices & bit) return hipSuccess;
   e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-  if (e == hipSuccess && slot != nullptr) {
-    slot->kernel = kernel;
-    slot->devices |= bit;
-  }
+  if (e == hipSuccess) devices |= bit;
   return e;
 }
 

@@ -536,9 +536,11 @@ def main():
         extra["per_format_gemm"] = {"note": "c3's M, N and K with 3584 (E4M3: 3328) of the 4096 channels in one activation format, "
                                             "on the kernels c3 runs; peak = the same blended nominal formula", "rows": per_format}
 
-        # ------------------------------------------------------------ plans without E3M2 and / or E4M3 activations
+        # ------------------------------------------------------------ plans without one or two of the activation formats
+        # (the last three: pure E3M2 x E2M1 and E4M3 x E2M1 products, what matmul_host6 / matmul_host8 of the
+        # reference compute on their own, bench_fp6.cu:109-122 and bench_fp8.cu, and E3M2 + E4M3)
         partial = []
-        for knf, ksf, kof in ((4096, 0, 0), (3968, 0, 128), (2560, 1536, 0)):
+        for knf, ksf, kof in ((4096, 0, 0), (3968, 0, 128), (2560, 1536, 0), (0, 4096, 0), (0, 0, 4096), (0, 3968, 128)):
             aqf = abi.reorder_quantize_x(xd, idd, knf, ksf, kof)
             wqf = abi.reorder_quantize_w(wd, idd, knf, ksf, kof)
             wtf = abi.tile_weights(*wqf[:3])

@@ -48,6 +48,41 @@ def _stale(target: str, deps: list[str]) -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
+# Kernels whose loads and LDS copies are inline assembly that the compiler does not count: a register such a load
+# is still to fill must never be moved or spilled, so these kernels must compile without scratch memory.  (The
+# whole-tile GEMM is listed for speed: a spill inside its K loop costs more than anything else there.)
+NO_SCRATCH_KERNELS = ("mixed_gemm_decode_kernel", "reorder_quant_dma_kernel", "mixed_gemm_256_kernel",
+                      "mixed_gemm_256_tail_kernel")
+
+
+def _split_remarks(stderr: str) -> tuple[str, str]:
+    """(resource-usage remarks, everything else) of a hipcc run with -Rpass-analysis=kernel-resource-usage."""
+    remarks, other, skip = [], [], 0
+    for line in stderr.splitlines():
+        if "-Rpass-analysis=kernel-resource-usage" in line:
+            remarks.append(line)
+            skip = 2          # the source line and the caret that follow a remark
+        elif skip and ("remark" not in line) and (line.strip().startswith(("|", "^")) or "|" in line[:8]):
+            skip -= 1
+        else:
+            other.append(line)
+    return "\n".join(remarks), "\n".join(other)
+
+
+def _check_no_scratch(src: str, remarks: str) -> None:
+    import re
+    name, bad = None, []
+    for line in remarks.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and name and int(m.group(1)) and any(k in name for k in NO_SCRATCH_KERNELS):
+            bad.append(f"{name}: {m.group(1)} bytes of scratch per lane")
+    if bad:
+        raise RuntimeError(f"{os.path.basename(src)}: kernels that must not spill do:\n  " + "\n  ".join(bad))
+
+
 def _compile_and_link(sources: list[str], target: str, force: bool, verbose: bool) -> str:
     """One object per source, compiled side by side, then one link."""
     from concurrent.futures import ThreadPoolExecutor
@@ -61,10 +96,20 @@ def _compile_and_link(sources: list[str], target: str, force: bool, verbose: boo
     def compile_one(pair):
         src, obj = pair
         if force or _stale(obj, [src] + hdrs):
-            cmd = ["hipcc", *HIPCC_FLAGS, "-c", src, "-o", obj]
+            cmd = ["hipcc", *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj]
             if verbose:
                 print(" ".join(cmd), flush=True)
-            subprocess.check_call(cmd)
+            done = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+            remarks, other = _split_remarks(done.stderr)
+            if other.strip():
+                print(other, file=sys.stderr, flush=True)
+            if done.returncode != 0:
+                raise subprocess.CalledProcessError(done.returncode, cmd)
+            try:
+                _check_no_scratch(src, remarks)
+            except Exception:
+                os.remove(obj)
+                raise
 
     with ThreadPoolExecutor(max_workers=min(len(srcs), 6)) as pool:
         list(pool.map(compile_one, zip(srcs, objs)))

@@ -764,289 +764,6 @@ hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeS
   return hipGetLastError();
 }
 
-// ---------------------------------------------------------------------------
-// LDS-tiled kernel on v_mfma_scale_f32_32x32x64_f8f6f4.
-//
-// Geometry of that instruction (measured on gfx950): lane l supplies row
-// i = l % 32 of its operand; with g = l / 32,
-//   E2M1 / E3M2: the 32 consecutive K elements of block g of the 64-wide K step;
-//   E4M3:        K [16g, 16g+16) in registers 0-3, K [32+16g, 32+16g+16) in 4-7;
-//   scale:       the E8M0 byte of (row i, block g), selected by op_sel;
-//   result:      column l % 32, rows 8*(v/4) + 4*g + v%4 for v = 0..15.
-//
-// Workgroup = 4 waves = 256 features x 128 tokens; wave = 128 x 64 (4 x 2 MFMA
-// tiles, 128 accumulator registers), two workgroups per CU so one covers the
-// other's barrier and memory stalls.  One K stage = 128 elements = one dword of
-// scales per row = two MFMA K steps; LDS is double buffered.
-//
-// Every operand byte goes global -> LDS directly (global_load_lds_dwordx4: no
-// staging registers, no LDS store instructions).  One such instruction moves
-// 64 x 16 B to 1 KB of consecutive LDS; each lane quad reads 64 (or 96)
-// contiguous bytes of one row.  Which rows an instruction gathers, and where its
-// block sits, is chosen so that the 16 lanes that fetch rows 32t..32t+15 of a
-// fragment land in 16 different banks groups:
-//   weights (64 B rows):  instruction j moves rows j, j+16, ..., j+240; block j
-//                         at j*1040, so those lanes are 65 slots of 16 B apart;
-//   E2M1 / E4M3 tokens:   instruction j moves rows j + 8t, t = 0..15, row t at
-//                         quad 4*(t/4) + tau(t%4), tau = (0,2,1,3); block j at
-//                         j*1040 (E4M3: one set of blocks per 64-wide K half);
-//   E3M2 tokens (96 B):   three instructions move rows j + 4t, t = 0..31, as one
-//                         row-major block of 3072 B at j*3088.
-// The scale atoms (512 B per 128 rows per stage) are copied the same way.
-// ---------------------------------------------------------------------------
-constexpr int kTileN = 256, kTileM = 128, kStageK = 128;
-constexpr int kBlock = 1040;                   // 16 rows x 64 B + 16 B of padding
-constexpr int kWBytes = 16 * kBlock;           // weights, E2M1: 64 B per row per stage
-constexpr int kXBytes = 16 * kBlock;           // activations, E4M3 worst case (E3M2: 4 * 3088)
-constexpr int kSBytes = 1024 + 512;            // two weight scale atoms + one activation scale atom
-constexpr int kStageBytes = kWBytes + kXBytes + kSBytes;
-
-struct Seg {
-  const uint8_t* a;    // activation codes of the segment
-  const uint8_t* b;    // weight codes
-  const uint8_t* sfa;  // activation scales
-  const uint8_t* sfb;  // weight scales
-  int stages;          // kseg / 128
-};
-
-template <int FMT> struct RowBytes;   // activation bytes per row per 128-wide stage
-template <> struct RowBytes<kFmtE2M1> { static constexpr int v = 64; };
-template <> struct RowBytes<kFmtE3M2> { static constexpr int v = 96; };
-template <> struct RowBytes<kFmtE4M3> { static constexpr int v = 128; };
-
-typedef int v6i __attribute__((ext_vector_type(6)));
-template <int FMT> struct XFrag;      // registers of one activation fragment
-template <> struct XFrag<kFmtE2M1> { typedef v4i type; };
-template <> struct XFrag<kFmtE3M2> { typedef v6i type; };
-template <> struct XFrag<kFmtE4M3> { typedef v8i type; };
-
-__device__ __forceinline__ v8i widen(v4i v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1); }
-__device__ __forceinline__ v8i widen(v6i v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3, 4, 5, -1, -1); }
-__device__ __forceinline__ v8i widen(v8i v) { return v; }
-
-typedef __attribute__((address_space(3))) void* lds_ptr;
-
-__device__ __forceinline__ void copy16(const uint8_t* base, unsigned off, uint8_t* lds_dst) {
-  __builtin_amdgcn_global_load_lds(base + off, (lds_ptr)lds_dst, 16, 0, 0);
-}
-
-__device__ __forceinline__ int tau(int e) { return ((e & 1) << 1) | (e >> 1); }   // (0,2,1,3)
-
-// Per-lane byte offsets into the operand rows, fixed for a segment.
-template <int FMT>
-struct CopyOffsets {
-  unsigned w, x[3], s;
-  __device__ __forceinline__ CopyOffsets(const Seg& sg, int lane) {
-    const unsigned ldb = (unsigned)sg.stages * 64, lda = (unsigned)sg.stages * RowBytes<FMT>::v;
-    const int p = lane >> 2, c = lane & 3;
-    w = (unsigned)(16 * p) * ldb + c * 16;
-    if constexpr (FMT == kFmtE3M2) {
-#pragma unroll
-      for (int k = 0; k < 3; ++k) {
-        const int ci = 64 * k + lane;
-        x[k] = (unsigned)(4 * (ci / 6)) * lda + (ci % 6) * 16;
-      }
-    } else {
-      const int t = 4 * (p >> 2) + tau(p & 3);
-      x[0] = (unsigned)(8 * t) * lda + c * 16;
-    }
-    s = (unsigned)(lane >> 5) * sg.stages * 512 + (lane & 31) * 16;
-  }
-};
-
-// Issue the copies of K stage q of a segment into LDS buffer `buf`.  `wave` is uniform.
-template <int FMT>
-__device__ __forceinline__ void stage_copy(const Seg& sg, const CopyOffsets<FMT>& off, int q, int n0, int m0,
-                                           uint8_t* buf, int wave, int lane) {
-  constexpr int RB = RowBytes<FMT>::v;
-  const unsigned ldb = (unsigned)sg.stages * 64, lda = (unsigned)sg.stages * RB;
-  const uint8_t* wbase = sg.b + (size_t)n0 * ldb + (size_t)q * 64;
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int j = wave * 4 + k;
-    copy16(wbase + (size_t)j * ldb, off.w, buf + j * kBlock);
-  }
-  const uint8_t* xbase = sg.a + (size_t)m0 * lda + (size_t)q * RB;
-  uint8_t* xb = buf + kWBytes;
-  if constexpr (FMT == kFmtE2M1) {
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      const int j = wave * 2 + k;
-      copy16(xbase + (size_t)j * lda, off.x[0], xb + j * kBlock);
-    }
-  } else if constexpr (FMT == kFmtE3M2) {
-#pragma unroll
-    for (int k = 0; k < 3; ++k) copy16(xbase + (size_t)wave * lda, off.x[k], xb + wave * 3088 + k * 1024);
-  } else {
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int id = wave * 4 + k, hh = id >> 3, j = id & 7;   // K half, row residue
-      copy16(xbase + (size_t)j * lda + hh * 64, off.x[0], xb + id * kBlock);
-    }
-  }
-  uint8_t* sb = buf + kWBytes + kXBytes;
-  if (wave == 0) {
-    copy16(sg.sfb + ((size_t)(n0 >> 7) * sg.stages + q) * 512, off.s, sb);
-  } else if (wave == 1) {
-    if (lane < 32) copy16(sg.sfa + ((size_t)(m0 >> 7) * sg.stages + q) * 512, off.s, sb + 1024);
-  }
-}
-
-// all fragments and scales of one stage: LDS -> registers
-template <int FMT>
-__device__ __forceinline__ void frags_read(v4i (&wf)[2][4], typename XFrag<FMT>::type (&xf)[2][2], v4i& sw, v4i& sx,
-                                           const uint8_t* __restrict__ buf, int lane, int wn, int wm) {
-  const int i = lane & 31, g = lane >> 5;
-  // row 32*rt + i of the weight tile: block i%16, quad 2*rt + i/16
-  const uint8_t* wl = buf + (i & 15) * kBlock + (i >> 4) * 64 + g * 16 + wn * 4 * 128;
-  const uint8_t* xb = buf + kWBytes;
-  const uint8_t* sb = buf + kWBytes + kXBytes;
-  sw = *reinterpret_cast<const v4i*>(sb + wn * 512 + i * 16);
-  sx = *reinterpret_cast<const v4i*>(sb + 1024 + i * 16);
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-#pragma unroll
-    for (int t = 0; t < 4; ++t) wf[h][t] = *reinterpret_cast<const v4i*>(wl + t * 128 + h * 32);
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int rt = wm * 2 + t;
-      if constexpr (FMT == kFmtE2M1) {
-        // row 32*rt + i: block i%8, quad 4*rt + tau(i/8)
-        xf[h][t] = *reinterpret_cast<const v4i*>(xb + (i & 7) * kBlock + (4 * rt + tau(i >> 3)) * 64 + (2 * h + g) * 16);
-      } else if constexpr (FMT == kFmtE3M2) {
-        // row 32*rt + i: block i%4, row slot 8*rt + i/4, fragment 2h+g of 24 bytes
-        const v2i* p = reinterpret_cast<const v2i*>(xb + (i & 3) * 3088 + (8 * rt + (i >> 2)) * 96 + (2 * h + g) * 24);
-        const v2i a = p[0], b = p[1], c = p[2];
-        xf[h][t] = v6i{a[0], a[1], b[0], b[1], c[0], c[1]};
-      } else {
-        const uint8_t* p = xb + (h * 8 + (i & 7)) * kBlock + (4 * rt + tau(i >> 3)) * 64 + g * 16;
-        const v4i a = *reinterpret_cast<const v4i*>(p);        // K [16g, 16g+16) of the half
-        const v4i b = *reinterpret_cast<const v4i*>(p + 32);   // K [32+16g, 32+16g+16)
-        xf[h][t] = v8i{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
-      }
-    }
-  }
-}
-
-template <int FMT>
-__device__ __forceinline__ void stage_compute(v16f (&acc)[4][2], const v4i (&wf)[2][4],
-                                              const typename XFrag<FMT>::type (&xf)[2][2], v4i sw, v4i sx, int lane,
-                                              int wm) {
-  const int g8 = (lane >> 5) * 8;
-  int scw[4], scx[2];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) scw[t] = (int)((unsigned)sw[t] >> g8);
-#pragma unroll
-  for (int t = 0; t < 2; ++t) scx[t] = (int)((unsigned)(wm ? sx[2 + t] : sx[t]) >> g8);
-#pragma unroll
-  for (int h = 0; h < 2; ++h)
-#pragma unroll
-    for (int tn = 0; tn < 4; ++tn)
-#pragma unroll
-      for (int tm = 0; tm < 2; ++tm) {
-        if (h == 0)
-          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(widen(wf[0][tn]), widen(xf[0][tm]), acc[tn][tm],
-                                                                        kFmtE2M1, FMT, 0, scw[tn], 0, scx[tm]);
-        else
-          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(widen(wf[1][tn]), widen(xf[1][tm]), acc[tn][tm],
-                                                                        kFmtE2M1, FMT, 2, scw[tn], 2, scx[tm]);
-      }
-}
-
-// Runs the stages of one segment.  While stage q is computed from one LDS buffer the copies
-// of stage q+1 (of this segment, or stage 0 of the next one) fill the other.  `pos` counts
-// stages across segments; LDS buffer = pos & 1.
-template <int FMT, int FMT_NEXT>
-__device__ __forceinline__ void segment_tiled(v16f (&acc)[4][2], const Seg& sg, const Seg& next, uint8_t* __restrict__ lds,
-                                              int& pos, int n0, int m0, int lane, int wave, int wn, int wm) {
-  if (sg.stages == 0) return;
-  const CopyOffsets<FMT> off(sg, lane);
-  for (int q = 0; q < sg.stages; ++q, ++pos) {
-    uint8_t* cur = lds + (pos & 1) * kStageBytes;
-    uint8_t* nxt = lds + ((pos + 1) & 1) * kStageBytes;
-    // this wave's copies for the current stage have landed; after the barrier everybody's have,
-    // and nobody still reads the other buffer
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-    __syncthreads();
-    v4i wf[2][4], sw, sx;
-    typename XFrag<FMT>::type xf[2][2];
-    frags_read<FMT>(wf, xf, sw, sx, cur, lane, wn, wm);
-    if (q + 1 < sg.stages) {
-      stage_copy<FMT>(sg, off, q + 1, n0, m0, nxt, wave, lane);
-    } else if (next.stages > 0) {
-      const CopyOffsets<FMT_NEXT> noff(next, lane);
-      stage_copy<FMT_NEXT>(next, noff, 0, n0, m0, nxt, wave, lane);
-    }
-    stage_compute<FMT>(acc, wf, xf, sw, sx, lane, wm);
-  }
-}
-
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
-mixed_gemm_tiled_kernel(Seg s4, Seg s6, Seg s8, int M, int N, uint16_t* __restrict__ d) {
-  extern __shared__ __align__(16) uint8_t lds[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wn = wave & 1, wm = wave >> 1;
-  const int n0 = blockIdx.x * kTileN, m0 = blockIdx.y * kTileM;
-
-  v16f acc[4][2];
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.0f;
-
-  int pos = 0;
-  const Seg none = {nullptr, nullptr, nullptr, nullptr, 0};
-  // an empty middle segment is skipped by handing its successor to the one before it
-  const Seg& after4 = s6.stages > 0 ? s6 : s8;
-  // first stage of the first non-empty segment
-  if (s4.stages > 0) stage_copy<kFmtE2M1>(s4, CopyOffsets<kFmtE2M1>(s4, lane), 0, n0, m0, lds, wave, lane);
-  else if (s6.stages > 0) stage_copy<kFmtE3M2>(s6, CopyOffsets<kFmtE3M2>(s6, lane), 0, n0, m0, lds, wave, lane);
-  else stage_copy<kFmtE4M3>(s8, CopyOffsets<kFmtE4M3>(s8, lane), 0, n0, m0, lds, wave, lane);
-
-  if (s6.stages > 0) segment_tiled<kFmtE2M1, kFmtE3M2>(acc, s4, after4, lds, pos, n0, m0, lane, wave, wn, wm);
-  else               segment_tiled<kFmtE2M1, kFmtE4M3>(acc, s4, after4, lds, pos, n0, m0, lane, wave, wn, wm);
-  segment_tiled<kFmtE3M2, kFmtE4M3>(acc, s6, s8, lds, pos, n0, m0, lane, wave, wn, wm);
-  segment_tiled<kFmtE4M3, kFmtE4M3>(acc, s8, none, lds, pos, n0, m0, lane, wave, wn, wm);
-
-  // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.
-  // Written straight from that layout a store instruction would touch 32 rows with 16 bytes each;
-  // instead each wave transposes its 64 tokens x 128 features through its own quarter of the (now
-  // idle) LDS, so that a store instruction writes 4 rows x 256 contiguous bytes.
-  constexpr int kPitch = 256 + 16;   // bytes per token row in LDS
-  static_assert(4 * 64 * kPitch <= 2 * kStageBytes, "epilogue staging must fit the stage buffers");
-  __syncthreads();                   // every wave is done with the last stage's fragments
-  uint8_t* stage = lds + wave * 64 * kPitch;
-  {
-    const int g = lane >> 5;
-    uint8_t* wr = stage + (lane & 31) * kPitch + 8 * g;
-#pragma unroll
-    for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-      for (int tn = 0; tn < 4; ++tn)
-#pragma unroll
-        for (int vq = 0; vq < 4; ++vq) {
-          const v2bf lo = {(__bf16)acc[tn][tm][4 * vq + 0], (__bf16)acc[tn][tm][4 * vq + 1]};
-          const v2bf hi = {(__bf16)acc[tn][tm][4 * vq + 2], (__bf16)acc[tn][tm][4 * vq + 3]};
-          *reinterpret_cast<v2u*>(wr + tm * 32 * kPitch + tn * 64 + vq * 16) =
-              v2u{__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
-        }
-  }
-  // only this wave reads what it wrote: no workgroup barrier needed
-  {
-    const int r = lane >> 4, c = lane & 15;
-    const uint8_t* rd = stage + r * kPitch + c * 16;
-    uint16_t* out = d + (size_t)(m0 + wm * 64 + r) * N + n0 + wn * 128 + c * 8;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const v4u v = *reinterpret_cast<const v4u*>(rd + i * 4 * kPitch);
-      *reinterpret_cast<v4u*>(out + (size_t)i * 4 * N) = v;
-    }
-  }
-}
-
 }  // namespace
 
 // 256 x 256 tiles, one workgroup per CU (mixed_gemm_256.hip)
@@ -1100,18 +817,8 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
   const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
   const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};
   if (M < 256 && KN + KS + KO > 0) return launch_skinny(d4, d6, d8, M, N, w_tiled, static_cast<uint16_t*>(d), stream);
-  // the tiled kernel needs whole tiles and whole 128-wide K stages
-  if (M % kTileM == 0 && N % kTileN == 0 && KN % kStageK == 0 && KS % kStageK == 0 && KO % kStageK == 0 &&
-      KN + KS + KO > 0) {
-    hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(mixed_gemm_tiled_kernel), 2 * kStageBytes);
-    if (e != hipSuccess) return e;
-    const Seg s4 = {an, bn, sfan, sfbn, KN / kStageK};
-    const Seg s6 = {as_, bs, sfas, sfbs, KS / kStageK};
-    const Seg s8 = {ao, bo, sfao, sfbo, KO / kStageK};
-    hipLaunchKernelGGL(mixed_gemm_tiled_kernel, dim3(N / kTileN, M / kTileM), dim3(256), 2 * kStageBytes, stream, s4, s6,
-                       s8, M, N, static_cast<uint16_t*>(d));
-    return hipGetLastError();
-  }
+  // what is left (256 tokens or more with N not a multiple of 8, or with a segment that is not whole 128-wide
+  // stages next to an empty one): the direct kernel
   dim3 grid(ceil_div(N, 64), ceil_div(M, 64));
   hipLaunchKernelGGL(mixed_gemm_direct_kernel, grid, dim3(256), 0, stream, an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs,
                      sfao, sfbo, M, N, KN, KS, KO, static_cast<uint16_t*>(d));

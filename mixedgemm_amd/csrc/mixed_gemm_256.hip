@@ -868,8 +868,23 @@ __device__ __forceinline__ Plan start_workgroup(const Plan& plan_arg, int first_
   return plan;
 }
 
+// Format of the k-th segment that exists in a plan (segs: bit 0 E2M1, bit 1 E3M2, bit 2 E4M3), kFmtNone past the last.
+constexpr int nth_format(int segs, int k) {
+  constexpr int fmts[3] = {kFmtE2M1, kFmtE3M2, kFmtE4M3};
+  for (int sg = 0; sg < 3; ++sg)
+    if (segs & (1 << sg)) {
+      if (k == 0) return fmts[sg];
+      --k;
+    }
+  return kFmtNone;
+}
+template <int FMT>
+__device__ __forceinline__ int stages_of(const Plan& p) {
+  return FMT == kFmtE2M1 ? p.st0 : (FMT == kFmtE3M2 ? p.st1 : (FMT == kFmtE4M3 ? p.st2 : 0));
+}
+
 // REGULAR: see run_segment.  REM: some segment is not a multiple of 128 wide.  WT: tile-major weights.
-// SEGS: which activation segments the plan has, bit 0 E2M1 (always), bit 1 E3M2, bit 2 E4M3 -- the
+// SEGS: which activation segments the plan has, bit 0 E2M1, bit 1 E3M2, bit 2 E4M3 -- the
 // prefetched fragments pass from a segment to the next one that exists, and their types are fixed here.
 // TM: token tiles of 32 per wave.  2: the workgroup's tile is 256 features x 256 tokens.  1: 256 x 128, for
 // problems with fewer than 256 whole tiles (every CU still gets a workgroup): same copies (the lanes of token
@@ -912,23 +927,25 @@ __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int t
   }
   // prologue: stages 0 and 1 and the first copies of stage 2 in flight; wait for stage 0 only.  The copies go out
   // before anything else that can wait (the accumulators are cleared while they are in flight); in REGULAR kernels
-  // the first three stages are E2M1 stages, or do not exist, and take the compile-time form of the copies.
-  const int n4 = plan.st0, n6 = plan.st1, n8 = plan.st2;
+  // the first three stages belong to the plan's first segment, or do not exist, and take the compile-time form of the copies.
+  constexpr int FA = nth_format(SEGS, 0), FB = nth_format(SEGS, 1), FC = nth_format(SEGS, 2);   // the segments that exist, in order
+  static_assert(FA != kFmtNone, "a plan has at least one segment");
+  const int nA = stages_of<FA>(plan), nB = stages_of<FB>(plan), nC = stages_of<FC>(plan);
   GenericCopy gc;
-  LeanCopy<kFmtE2M1, WT> l4;
+  LeanCopy<FA, WT> la;
   int in_flight;   // copies that may stay in flight while stage 0 is awaited
   if constexpr (REGULAR) {
-    l4.init(plan, 0, lo, c);
-    issue_range<0, kCopySlots>(l4, 0);
+    la.init(plan, 0, lo, c);
+    issue_range<0, kCopySlots>(la, 0);
     in_flight = 0;
     if (plan.total > 1) {
-      l4.advance();
-      issue_range<0, kCopySlots>(l4, kStage);
-      in_flight = l4.count();
+      la.advance();
+      issue_range<0, kCopySlots>(la, kStage);
+      in_flight = la.count();
     }
     if (plan.total > 2) {
-      l4.advance();   // stays on stage 2: where the segment loop expects it
-      issue_range<0, kSplit>(l4, 2 * kStage);
+      la.advance();   // stays on stage 2: where the segment loop expects it
+      issue_range<0, kSplit>(la, 2 * kStage);
       in_flight += kSplit;
     }
   } else {
@@ -942,11 +959,11 @@ __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int t
   }
   // the copy state of the later segments, while the first copies are in flight: set up between two halves of a
   // stage it would hold up the MFMAs for several hundred cycles
-  LeanCopy<kFmtE3M2, WT> l6;
-  LeanCopy<kFmtE4M3, WT> l8;
+  LeanCopy<FB, WT> lb;
+  LeanCopy<FC, WT> lcc;
   if constexpr (REGULAR) {
-    if constexpr ((SEGS & 2) != 0) l6.init(plan, n4, lo, c);
-    if constexpr ((SEGS & 4) != 0) l8.init(plan, n4 + n6, lo, c);
+    lb.init(plan, nA, lo, c);          // (no-ops for segments that do not exist)
+    lcc.init(plan, nA + nB, lo, c);
   }
   __builtin_amdgcn_sched_barrier(0);
 
@@ -980,32 +997,30 @@ __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int t
   wait_copies_but(in_flight);
   asm volatile("s_barrier" ::: "memory");
 
-  static_assert(SEGS == 7 || (REGULAR && !REM && (SEGS == 1 || SEGS == 3 || SEGS == 5)), "plans with an empty segment");
-  HalfFrags<kFmtE2M1, TM> a4, none4;
-  HalfFrags<kFmtE3M2, TM> a6, none6;
-  HalfFrags<kFmtE4M3, TM> a8, none;
+  static_assert(SEGS >= 1 && SEGS <= 7 && (SEGS == 7 || !REM), "plans with an empty segment: whole stages only");
+  HalfFrags<FA, TM> fa, da;   // d*: never-read targets of the prefetch past a plan's last stage
+  HalfFrags<FB, TM> fb, db;
+  HalfFrags<FC, TM> fc, dc;
   Scales<TM> sc;
   {
-    const TokenPtrs<kFmtE2M1, TM> xp(lds, c);
+    const TokenPtrs<FA, TM> xp(lds, c);
     v4i sw, sx;
-    const FragReader<kFmtE2M1, 0, true, TM> rd{a4, sw, sx, wp.w, xp.x, wp.sw, wp.sx, true};
+    const FragReader<FA, 0, true, TM> rd{fa, sw, sx, wp.w, xp.x, wp.sw, wp.sx, true};
     read_all(rd);
     wait_lds_reads();
     shift_scales(sc, sw, sx, c.lane, c.xtile);
   }
   LeanCopy<kFmtNone, WT> l0;
-  if constexpr (SEGS == 7) {
-    run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
-    run_segment<kFmtE3M2, kFmtE4M3, kFmtE4M3, REGULAR, NLAST>(acc, a6, sc, a8, l6, l8, gc, lo, plan, n6, n8, n4, wp, lds, c);
-    run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR, NLAST>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4 + n6, wp, lds, c);
-  } else if constexpr (SEGS == 5) {
-    run_segment<kFmtE2M1, kFmtE4M3, kFmtE4M3, REGULAR, NLAST>(acc, a4, sc, a8, l4, l8, gc, lo, plan, n4, n8, 0, wp, lds, c);
-    run_segment<kFmtE4M3, kFmtNone, kFmtE4M3, REGULAR, NLAST>(acc, a8, sc, none, l8, l0, gc, lo, plan, n8, 0, n4, wp, lds, c);
-  } else if constexpr (SEGS == 3) {
-    run_segment<kFmtE2M1, kFmtE3M2, kFmtE3M2, REGULAR, NLAST>(acc, a4, sc, a6, l4, l6, gc, lo, plan, n4, n6, 0, wp, lds, c);
-    run_segment<kFmtE3M2, kFmtNone, kFmtE3M2, REGULAR, NLAST>(acc, a6, sc, none6, l6, l0, gc, lo, plan, n6, 0, n4, wp, lds, c);
+  // NLAST goes to the plan's last segment and the one before it (see run_segment)
+  if constexpr (FB == kFmtNone) {
+    run_segment<FA, kFmtNone, FA, REGULAR>(acc, fa, sc, da, la, l0, gc, lo, plan, nA, 0, 0, wp, lds, c);
+  } else if constexpr (FC == kFmtNone) {
+    run_segment<FA, FB, FB, REGULAR, NLAST>(acc, fa, sc, fb, la, lb, gc, lo, plan, nA, nB, 0, wp, lds, c);
+    run_segment<FB, kFmtNone, FB, REGULAR, NLAST>(acc, fb, sc, db, lb, l0, gc, lo, plan, nB, 0, nA, wp, lds, c);
   } else {
-    run_segment<kFmtE2M1, kFmtNone, kFmtE2M1, REGULAR>(acc, a4, sc, none4, l4, l0, gc, lo, plan, n4, 0, 0, wp, lds, c);
+    run_segment<FA, FB, FB, REGULAR>(acc, fa, sc, fb, la, lb, gc, lo, plan, nA, nB, 0, wp, lds, c);
+    run_segment<FB, FC, FC, REGULAR, NLAST>(acc, fb, sc, fc, lb, lcc, gc, lo, plan, nB, nC, nA, wp, lds, c);
+    run_segment<FC, kFmtNone, FC, REGULAR, NLAST>(acc, fc, sc, dc, lcc, l0, gc, lo, plan, nC, 0, nA + nB, wp, lds, c);
   }
 
   // Result tile is D^T: lane holds token m = lane % 32, features 8*(v/4) + 4*(lane/32) + v%4.
@@ -1108,13 +1123,9 @@ bool mixed_gemm_256_supported(int M, int N, int KN, int KS, int KO) {
   // all three segments with at least one whole 128-wide stage: the pipeline hands the prefetched
   // fragments from one segment's loop to the next, in the order E2M1 -> E3M2 -> E4M3
   if (KN >= 128 && KS >= 128 && KO >= 128) return true;
-  // plans without E3M2 and / or E4M3 activations: whole stages only, and three of them in every segment
-  // that is followed by another (the variants with compiled-in segment-boundary copies)
-  if ((KN | KS | KO) % 128 != 0 || KN < 128) return false;
-  if (KS == 0 && KO == 0) return true;
-  if (KS == 0) return KN >= 384;
-  if (KO == 0) return KN >= 384;
-  return false;
+  // plans without one or two of the segments (pure E3M2 x E2M1 and E4M3 x E2M1 products among them, the reference's
+  // matmul_host6 / matmul_host8 on their own): whole stages only
+  return (KN | KS | KO) % 128 == 0 && KN + KS + KO > 0;
 }
 
 // Token rows per workgroup tile for a problem of m_store tokens: 256, or 128 when the 256 x 256 tiles would leave
@@ -1128,22 +1139,29 @@ static int tile_tokens(int m_store, int N, int cus) {
 typedef void (*kernel_t)(Plan, int, int, int, int, uint16_t*, int, int);
 
 // The kernel for a plan: segs = which activation segments exist (bit 0 E2M1, 1 E3M2, 2 E4M3), nlast = stages of the
-// last one (3 = three or more).  Plans with an empty segment exist in the REGULAR, whole-stage form only.
+// last one (3 = three or more), regular = every segment but the last has at least three stages.  Plans with an empty
+// segment exist in the whole-stage form only (!REM).
+template <bool REM, bool WT, int TM, int SEGS>
+static kernel_t select_by_length(bool regular, int nlast) {
+  constexpr bool kOne = SEGS == 1 || SEGS == 2 || SEGS == 4;   // one segment: nothing to hand over, any length
+  if constexpr (kOne) return mixed_gemm_256_kernel<true, REM, WT, SEGS, TM, 0>;
+  if (!regular) return mixed_gemm_256_kernel<false, REM, WT, SEGS, TM, 0>;
+  return nlast == 1 ? mixed_gemm_256_kernel<true, REM, WT, SEGS, TM, 1>
+                    : (nlast == 2 ? mixed_gemm_256_kernel<true, REM, WT, SEGS, TM, 2> : mixed_gemm_256_kernel<true, REM, WT, SEGS, TM, 3>);
+}
 template <bool REM, bool WT, int TM>
 static kernel_t select_kernel(bool regular, int segs, int nlast) {
-  if (segs == 7) {
-    if (!regular) return mixed_gemm_256_kernel<false, REM, WT, 7, TM, 0>;
-    return nlast == 1 ? mixed_gemm_256_kernel<true, REM, WT, 7, TM, 1>
-                      : (nlast == 2 ? mixed_gemm_256_kernel<true, REM, WT, 7, TM, 2> : mixed_gemm_256_kernel<true, REM, WT, 7, TM, 3>);
-  }
+  if (segs == 7) return select_by_length<REM, WT, TM, 7>(regular, nlast);
   if constexpr (!REM) {
-    if (segs == 1) return mixed_gemm_256_kernel<true, false, WT, 1, TM, 0>;
-    if (segs == 3)
-      return nlast == 1 ? mixed_gemm_256_kernel<true, false, WT, 3, TM, 1>
-                        : (nlast == 2 ? mixed_gemm_256_kernel<true, false, WT, 3, TM, 2> : mixed_gemm_256_kernel<true, false, WT, 3, TM, 3>);
-    if (segs == 5)
-      return nlast == 1 ? mixed_gemm_256_kernel<true, false, WT, 5, TM, 1>
-                        : (nlast == 2 ? mixed_gemm_256_kernel<true, false, WT, 5, TM, 2> : mixed_gemm_256_kernel<true, false, WT, 5, TM, 3>);
+    switch (segs) {
+      case 1: return select_by_length<false, WT, TM, 1>(regular, nlast);
+      case 2: return select_by_length<false, WT, TM, 2>(regular, nlast);
+      case 3: return select_by_length<false, WT, TM, 3>(regular, nlast);
+      case 4: return select_by_length<false, WT, TM, 4>(regular, nlast);
+      case 5: return select_by_length<false, WT, TM, 5>(regular, nlast);
+      case 6: return select_by_length<false, WT, TM, 6>(regular, nlast);
+      default: break;
+    }
   }
   return nullptr;
 }
@@ -1168,11 +1186,11 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
   if (hipError_t e = device_limits(&lim); e != hipSuccess) return e;
   const int tokens = tile_tokens(m_store, N, lim.cus);
   const int M = (m_store + tokens - 1) / tokens * tokens;
-  // every segment but the last at least 3 stages: the copies across segment boundaries are compiled in
-  const bool regular = KN >= 384 && KS >= 384;   // whole stages: KN / 128 >= 3, KS / 128 >= 3
   const bool rem = (KN | KS | KO) % 128 != 0;
   const int half = tokens == 128 ? 1 : 0;
-  const int segs = 1 | (KS > 0 ? 2 : 0) | (KO > 0 ? 4 : 0);
+  const int segs = (KN > 0 ? 1 : 0) | (KS > 0 ? 2 : 0) | (KO > 0 ? 4 : 0);
+  // every segment that another follows has at least 3 whole stages: the copies across segment boundaries are compiled in
+  const bool regular = (KN == 0 || KN >= 384 || (KS == 0 && KO == 0)) && (KS == 0 || KS >= 384 || KO == 0);
   const int last_stages = KO > 0 ? KO / 128 : (KS > 0 ? KS / 128 : KN / 128);
   const int nlast = last_stages >= 3 ? 3 : last_stages;
   // token tiles of 32 per wave: 2 for 256 x 256 workgroup tiles, 1 for 256 x 128

@@ -77,14 +77,19 @@ def test_reference_benchmark_shape(abi):
     _run_and_check(abi, m, n, kn, ks, ko, 8123, "reference bench shape")
 
 
-@pytest.mark.parametrize("m,n,k", [(4096, 4096, 12288), (2048, 3584, 18944)])
-def test_long_k_rows_of_the_shape_matrix_sampled(abi, m, n, k):
-    """Two rows of bench.py's shape matrix at (close to) full size: tile-major weights, sampled token rows
+@pytest.mark.parametrize("m,n,k,split", [
+    (4096, 4096, 12288, None), (2048, 3584, 18944, None),
+    # c3's M, N and K as pure E3M2 x E2M1 and E4M3 x E2M1 products (matmul_host6 / matmul_host8 of the reference on
+    # their own: src/fp6.cu:35, src/fp8.cu:35) and without the E2M1 segment: the legs of bench.py's plans_without_a_segment
+    (4096, 14336, 4096, (0, 4096, 0)), (4096, 14336, 4096, (0, 0, 4096)), (4096, 14336, 4096, (0, 3968, 128)),
+])
+def test_long_k_rows_of_the_shape_matrix_sampled(abi, m, n, k, split):
+    """Rows of bench.py's shape matrix at (close to) full size: tile-major weights, sampled token rows
     against the oracle, every tile through the permutation property."""
     from mixedgemm_amd.linear import default_split
     from oracle import mx_oracle as mo
-    kn, ks, ko = default_split(k)
-    _say("shape matrix row", m, n, k)
+    kn, ks, ko = split or default_split(k)
+    _say("shape matrix row", m, n, k, (kn, ks, ko))
     x = H.make_activations(m, k, 911 + k)
     w = H.make_weights(n, k, 913 + k)
     idx = H.absmax_sort_index(x)

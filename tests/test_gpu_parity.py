@@ -160,10 +160,10 @@ GEMM_SHAPES = [
     (20, 64, 448, 224, 64), (1, 16, 32, 32, 32),
     # decode kernel (M <= 16): ragged N, partial K steps, more K steps than one pass keeps in flight
     (8, 200, 96, 160, 64), (3, 1000, 2560, 1408, 128), (16, 48, 8192, 4096, 1024), (5, 40, 0, 4928, 448),
-    # whole 128 x 256 tiles and 128-wide K stages: the LDS-tiled kernel
+    # 128 tokens x 256 features and whole 128-wide K stages (the skinny kernel, or 256 x 128 tiles where they are estimated faster)
     (128, 256, 256, 0, 0), (128, 256, 0, 256, 0), (128, 256, 0, 0, 128), (128, 256, 128, 0, 128),
     (256, 512, 384, 256, 128), (128, 256, 2560, 1408, 128), (384, 768, 1280, 640, 128),
-    # whole 256 x 256 tiles with all three segments: the one-workgroup-per-CU kernel
+    # whole tiles with all three segments: the one-workgroup-per-CU kernel
     (256, 256, 128, 128, 128), (512, 256, 256, 384, 128), (256, 768, 2560, 1408, 128), (512, 512, 640, 256, 256),
     # the same with at least three 128-wide stages in the first two segments (segment-boundary copies compiled in)
     (256, 256, 384, 384, 384), (512, 256, 512, 384, 128), (256, 512, 384, 512, 256),
@@ -181,8 +181,12 @@ GEMM_SHAPES = [
     # weight row again and store only the pieces that exist
     (300, 1000, 2560, 1408, 128), (256, 264, 384, 384, 384), (512, 136, 448, 416, 224), (700, 8, 128, 128, 128),
     (256, 392, 512, 0, 0), (384, 648, 384, 0, 128),
-    # 256 or more tokens with another empty segment: the LDS-tiled kernel
-    (256, 256, 256, 0, 0), (384, 256, 0, 256, 128), (256, 512, 128, 0, 128),
+    # plans without E2M1 activations on the whole-tile kernel: pure E3M2 x E2M1 and E4M3 x E2M1 products (the reference's
+    # matmul_host6 / matmul_host8 alone), E3M2 + E4M3 with and without three stages in the first of them; and plans
+    # whose first segment is shorter than three stages next to an empty one (run-time segment-boundary copies)
+    (256, 256, 0, 256, 0), (512, 256, 0, 1024, 0), (300, 264, 0, 128, 0), (256, 256, 0, 0, 128), (256, 512, 0, 0, 640),
+    (256, 256, 0, 384, 128), (300, 512, 0, 512, 384), (384, 256, 0, 256, 128), (256, 256, 0, 128, 256),
+    (256, 256, 256, 0, 0), (256, 512, 128, 0, 128), (256, 256, 256, 128, 0), (512, 256, 128, 256, 0),
 ]
 
 
@@ -237,6 +241,8 @@ BIG_TILE_SHAPES = [
     (2304, 3840, 384, 384, 128), (2304, 3840, 384, 384, 256), (2304, 3840, 384, 384, 384), (2304, 3840, 448, 416, 224),
     (2304, 3840, 512, 0, 0), (2304, 3840, 384, 128, 0), (2304, 3840, 384, 256, 0), (2304, 3840, 384, 0, 128),
     (2304, 3840, 384, 0, 384), (2100, 3848, 384, 384, 128),
+    # plans without E2M1 activations, and two-segment plans with a short first segment (tile-major weights as well)
+    (2304, 3840, 0, 512, 0), (2304, 3840, 0, 0, 256), (2304, 3840, 0, 384, 128), (2304, 3840, 0, 256, 256), (2304, 3840, 256, 0, 128),
     # 1, 2 and 3 blocks of 32 past the whole stages in every segment (computed ahead of the K loop, absent K halves
     # skipped), with and without compiled-in segment boundaries, ragged tokens and features
     (2304, 3840, 416, 480, 160), (2304, 3840, 480, 448, 192), (2304, 3840, 160, 224, 352), (2100, 3848, 480, 448, 192),
@@ -687,9 +693,11 @@ def test_tiled_flag_is_refused_for_shapes_that_cannot_be_tiled(abi):
 # ------------------------------------------------------------------ RMSNorm fused into the quantizer
 @pytest.mark.parametrize("rows,kn,ks,ko,eps", [
     (7, 2560, 1408, 128, 1e-5), (130, 2560, 896, 128, 1e-6), (5, 128, 64, 64, 0.0),
-    (9, 8960, 4928, 448, 1e-5),      # two rows per pass
-    (3, 11776, 6560, 608, 1e-5),     # K = 18944: 1024-lane workgroups
-    (1030, 256, 128, 128, 1e-5),     # more row groups than resident workgroups: streamed
+    (9, 8960, 4928, 448, 1e-5),      # K = 14336: one lane per block, 448-lane workgroups
+    (3, 11776, 6560, 608, 1e-5),     # K = 18944: 640-lane workgroups
+    (1030, 256, 128, 128, 1e-5),     # more rows than resident workgroups: several rows per workgroup
+    (5, 20480, 11264, 992, 1e-5),    # K = 32736, the largest: the kernel with a run-time workgroup size (1024 lanes)
+    (300, 15360, 8448, 768, 1e-6),   # K = 24576 on the same kernel, two rows per workgroup for some
 ])
 def test_rmsnorm_reorder_quantize_matches_oracle(abi, rows, kn, ks, ko, eps):
     k = kn + ks + ko
@@ -705,8 +713,11 @@ def test_rmsnorm_reorder_quantize_matches_oracle(abi, rows, kn, ks, ko, eps):
     H.assert_quant_equal(got, want, rows, (kn, ks, ko), what=f"norm x {rows}x{k}")
 
 
-def test_fused_norm_linear_equals_norm_then_linear(abi):
-    m, n, kn, ks, ko, eps = 300, 512, 2560, 1408, 128, 1e-5
+@pytest.mark.parametrize("m,n,kn,ks,ko,eps", [
+    (300, 512, 2560, 1408, 128, 1e-5),
+    (40, 256, 15360, 8448, 768, 1e-5),    # K = 24576: the quantizer with a run-time workgroup size
+])
+def test_fused_norm_linear_equals_norm_then_linear(abi, m, n, kn, ks, ko, eps):
     k = kn + ks + ko
     x = H.make_activations(m, k, 61)
     w = H.make_weights(n, k, 62)

@@ -55,6 +55,11 @@ NO_SCRATCH_KERNELS = ("mixed_gemm_decode_kernel", "reorder_quant_dma_kernel", "m
                       "mixed_gemm_256_tail_kernel")
 
 
+# ... except the quantizer for K > 20480 (run-time workgroup size, up to 1024 lanes of 128 registers): it spills, and
+# reads its index and its gathered channels through loads the compiler sees instead.
+MAY_SPILL = ("reorder_quant_dma_kernelILi32ELi0E",)
+
+
 def _split_remarks(stderr: str) -> tuple[str, str]:
     """(resource-usage remarks, everything else) of a hipcc run with -Rpass-analysis=kernel-resource-usage."""
     remarks, other, skip = [], [], 0
@@ -77,7 +82,7 @@ def _check_no_scratch(src: str, remarks: str) -> None:
         if m:
             name = m.group(1)
         m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
-        if m and name and int(m.group(1)) and any(k in name for k in NO_SCRATCH_KERNELS):
+        if m and name and int(m.group(1)) and any(k in name for k in NO_SCRATCH_KERNELS) and not any(k in name for k in MAY_SPILL):
             bad.append(f"{name}: {m.group(1)} bytes of scratch per lane")
     if bad:
         raise RuntimeError(f"{os.path.basename(src)}: kernels that must not spill do:\n  " + "\n  ".join(bad))

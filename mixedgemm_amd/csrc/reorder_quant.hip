@@ -195,13 +195,19 @@ __device__ __forceinline__ void wait_vm(int n) {
   }
 }
 
-// 16 gathered channels: u[p] <- bf16 at LDS address ga[p] (+ OFF as an immediate, or + add), as the upper half
+// 16 gathered channels: u[p] <- bf16 at LDS address ga[p] + OFF (an immediate), as the upper half.  OFF < 0 (the
+// kernel with a run-time workgroup size, 1024 lanes and 128 registers each, which spills): at ga[p] + add, through
+// reads the compiler sees and waits for itself, so that a spilled register is always a loaded one.
 template <int OFF>
 __device__ __forceinline__ void gather16(unsigned (&u)[16], const unsigned (&ga)[16], unsigned add) {
 #pragma unroll
   for (int p = 0; p < 16; ++p) {
-    if constexpr (OFF >= 0) asm volatile("ds_read_u16_d16_hi %0, %1 offset:%2" : "+v"(u[p]) : "v"(ga[p]), "n"(OFF));
-    else asm volatile("ds_read_u16_d16_hi %0, %1" : "+v"(u[p]) : "v"(ga[p] + add));
+    if constexpr (OFF >= 0) {
+      asm volatile("ds_read_u16_d16_hi %0, %1 offset:%2" : "+v"(u[p]) : "v"(ga[p]), "n"(OFF));
+    } else {
+      typedef __attribute__((address_space(3))) const uint16_t* lds_u16;
+      u[p] = (unsigned)*reinterpret_cast<lds_u16>((size_t)(ga[p] + add)) << 16;
+    }
   }
 }
 // the reads above are invisible to the compiler's own wait insertion: wait here, with the registers tied to the wait
@@ -352,8 +358,13 @@ reorder_quant_dma_kernel(const uint8_t* __restrict__ x, const int16_t* __restric
   v4u iv[kPieces];
   {
     const v4u* ip = reinterpret_cast<const v4u*>(idx + (size_t)(has_block ? b : 0) * 32 + half * 16);
+    // (kernels with a compile-time workgroup size: as uncounted loads, waited for below; they compile without scratch
+    // memory -- the build checks it --, so that no register is moved before its load has landed)
 #pragma unroll
-    for (int q = 0; q < kPieces; ++q) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(iv[q]) : "v"(ip + q) : "memory");
+    for (int q = 0; q < kPieces; ++q) {
+      if constexpr (kImm) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(iv[q]) : "v"(ip + q) : "memory");
+      else iv[q] = ip[q];
+    }
   }
 #pragma unroll
   for (int s = 0; s < NS; ++s)
@@ -420,7 +431,7 @@ reorder_quant_dma_kernel(const uint8_t* __restrict__ x, const int16_t* __restric
       // bit of a double, which the rounding to fp32 all but never sees).  A lane works on the pieces it copied.
       uint8_t* slot = lds + S * stride;
       v4u a[kPieces];
-      double ss = 0.0;
+      double part[4] = {0.0, 0.0, 0.0, 0.0};   // four chains: one chain of dependent fp64 fmas would wait for each in turn
 #pragma unroll
       for (int it = 0; it < kPieces; ++it) {
         a[it] = *reinterpret_cast<const v4u*>(slot + (size_t)(it * nthr + tid) * 16);
@@ -429,12 +440,12 @@ reorder_quant_dma_kernel(const uint8_t* __restrict__ x, const int16_t* __restric
           for (int e = 0; e < 4; ++e) {
             const unsigned d = a[it][e];
             const double lo = (double)__uint_as_float(d << 16), hi = (double)__uint_as_float(d & 0xffff0000u);
-            ss = __builtin_fma(lo, lo, ss);
-            ss = __builtin_fma(hi, hi, ss);
+            part[e] = __builtin_fma(lo, lo, part[e]);
+            part[e] = __builtin_fma(hi, hi, part[e]);
           }
         }
       }
-      ss = wave_sum(ss);
+      double ss = wave_sum((part[0] + part[1]) + (part[2] + part[3]));
       if ((tid & 63) == 0) row_sums[i & 1][tid >> 6] = ss;
       __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the sum is in the LDS (a raw barrier implies no wait of the compiler's)
       asm volatile("s_barrier" ::: "memory");   // also: every wave's copies of row i have landed, every wave is past its gather of row i - 1

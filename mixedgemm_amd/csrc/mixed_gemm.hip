@@ -326,7 +326,8 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
 }
 
 // ---------------------------------------------------------------------------
-// Decode kernel: up to 16 tokens, whole 128-wide K steps.
+// Decode kernel: 16 G tokens per workgroup (G = 1: up to 16 tokens in all; G = 2: up to 255 tokens, 32 per workgroup,
+// where their codes fit the LDS), whole 128-wide K steps.
 //
 // The skinny kernel above issues seven loads per K step and wave, five of them for a few bytes each (the
 // token fragment twice, three scale bytes); the address unit handles those as slowly as the two 1 KB weight
@@ -349,11 +350,11 @@ mixed_gemm_skinny_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
 // ---------------------------------------------------------------------------
 struct DecodeLds {
   int x0, x1, x2;        // byte offsets of the token codes per segment
-  int sfa0, sfa1, sfa2;  // of the token scale pieces: per step pa pieces of 16 bytes (tokens 0 .. pa - 1)
+  int sfa0, sfa1, sfa2;  // of the token scale pieces: per step pa pieces of 16 bytes (piece p: tokens p, p + 32, p + 64, p + 96 of a group of 128)
   int sfb0, sfb1, sfb2;  // of the weight scale pieces: per step 4 F pieces
   int partial;           // of the partial sums
   int total;
-  int pa;                // 8 (up to 8 tokens) or 16
+  int pa;                // 8 (up to 8 tokens), 16, or 32 (G = 2: the whole atom of the workgroup's group of 128 tokens)
 };
 
 // value of segment seg (0, 1, 2) by masking: a select between struct fields invites the compiler to index a private
@@ -429,10 +430,11 @@ __device__ __forceinline__ void tie(v4i& r) { asm volatile("" : "+v"(r)); }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
 
-template <int F, bool WT>
+template <int F, bool WT, int G>
 __global__ void __launch_bounds__(256)
 mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N, int steps_per_wave, DecodeLds L,
                          uint16_t* __restrict__ d) {
+  static_assert(G == 1 || G == 2, "token groups of 16 per workgroup");
   constexpr int S = 4;        // K steps per round
   constexpr int PB = 4 * F;   // weight scale pieces per step
   constexpr int PBLOG = F == 1 ? 2 : (F == 2 ? 3 : 4);
@@ -524,15 +526,20 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
   };
   // ---- what is not a weight code, into LDS: requested first (measured: with the first round of weights ahead of
   // them the kernel is slower, by 2 % on tile-major and 7 % on row-major weights)
-  copy_region(s4.a, M * nblk4 * 16, lds0 + L.x0, wave, lane);
-  copy_region(s6.a, M * nblk6 * 24, lds0 + L.x1, wave, lane);
-  copy_region(s8.a, M * nblk8 * 32, lds0 + L.x2, wave, lane);
+  // the workgroup's tokens: m_base ... m_base + rows_here - 1 (G = 2: workgroup blockIdx.y takes 32 of them)
+  const int m_base = G == 1 ? 0 : (int)blockIdx.y * 32;
+  const int rows_here = min(M - m_base, 16 * G);
+  copy_region(s4.a + (size_t)m_base * nblk4 * 16, rows_here * nblk4 * 16, lds0 + L.x0, wave, lane);
+  copy_region(s6.a + (size_t)m_base * nblk6 * 24, rows_here * nblk6 * 24, lds0 + L.x1, wave, lane);
+  copy_region(s8.a + (size_t)m_base * nblk8 * 32, rows_here * nblk8 * 32, lds0 + L.x2, wave, lane);
   {
-    const int palog = L.pa == 8 ? 3 : 4;
-    const unsigned pa_off = (unsigned)(lane & (L.pa - 1)) * 16u;   // token scale pieces 0 ... pa - 1 of the first group of rows
-    if (s4.steps) copy_pieces(s4.sfa, s4.steps, palog, pa_off, lds0 + L.sfa0, wave, lane);
-    if (s6.steps) copy_pieces(s6.sfa, s6.steps, palog, pa_off, lds0 + L.sfa1, wave, lane);
-    if (s8.steps) copy_pieces(s8.sfa, s8.steps, palog, pa_off, lds0 + L.sfa2, wave, lane);
+    const int palog = L.pa == 8 ? 3 : (L.pa == 16 ? 4 : 5);
+    // token scale pieces 0 ... pa - 1 of the tokens' group of 128 rows
+    const unsigned pa_off = (unsigned)(lane & (L.pa - 1)) * 16u;
+    const unsigned agrp = (unsigned)(m_base >> 7) * 512u;   // times the segment's atoms along K
+    if (s4.steps) copy_pieces(s4.sfa, s4.steps, palog, pa_off + agrp * (unsigned)s4.steps, lds0 + L.sfa0, wave, lane);
+    if (s6.steps) copy_pieces(s6.sfa, s6.steps, palog, pa_off + agrp * (unsigned)s6.steps, lds0 + L.sfa1, wave, lane);
+    if (s8.steps) copy_pieces(s8.sfa, s8.steps, palog, pa_off + agrp * (unsigned)s8.steps, lds0 + L.sfa2, wave, lane);
     if (s4.steps) copy_pieces(s4.sfb, s4.steps, PBLOG, sfb_piece_off + (unsigned)(sfb_katoms_mul * s4.steps) * 512u, lds0 + L.sfb0, wave, lane);
     if (s6.steps) copy_pieces(s6.sfb, s6.steps, PBLOG, sfb_piece_off + (unsigned)(sfb_katoms_mul * s6.steps) * 512u, lds0 + L.sfb1, wave, lane);
     if (s8.steps) copy_pieces(s8.sfb, s8.steps, PBLOG, sfb_piece_off + (unsigned)(sfb_katoms_mul * s8.steps) * 512u, lds0 + L.sfb2, wave, lane);
@@ -546,10 +553,20 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
   else wait_vmcnt<0>();
   asm volatile("s_barrier" ::: "memory");
 
-  v4f acc[F];
+  v4f acc[F][G];
 #pragma unroll
-  for (int f = 0; f < F; ++f) acc[f] = v4f{0.f, 0.f, 0.f, 0.f};
-  const int mc = min(i, M - 1);   // token of this lane (tokens past M: the last one again, never stored)
+  for (int f = 0; f < F; ++f)
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) acc[f][gi] = v4f{0.f, 0.f, 0.f, 0.f};
+  // token of this lane in token group gi, as a row of the workgroup's LDS image (tokens past M: the last one again,
+  // never stored), and where its scale bytes sit in a step's pieces
+  int mc[G], sx_off[G];
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) {
+    mc[gi] = min(16 * gi + i, rows_here - 1);
+    const int mg = m_base + mc[gi];
+    sx_off[gi] = (mg & (L.pa - 1)) * 16 + ((mg >> 5) & 3) * 4;
+  }
   const int pa16 = L.pa * 16;
 
   auto compute_round = [&](int r, auto buf_c) {
@@ -562,7 +579,9 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
         const int q = seg == 0 ? t : (seg == 1 ? t - s4.steps : t - s4.steps - s6.steps);
         const uint8_t* sfa_l = lds + sel3(seg, L.sfa0, L.sfa1, L.sfa2) + q * pa16;
         const uint8_t* sfb_l = lds + sel3(seg, L.sfb0, L.sfb1, L.sfb2) + q * (PB * 16);
-        const int s_x = sfa_l[mc * 16 + g];
+        int s_x[G];
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi) s_x[gi] = sfa_l[sx_off[gi] + g];
         v8i wf[F];
         int s_w[F];
 #pragma unroll
@@ -571,23 +590,26 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
           const v4i w4 = wq[B][k][f];
           wf[f] = v8i{w4[0], w4[1], w4[2], w4[3], 0, 0, 0, 0};
         }
-        if (seg == 0) {
-          const v4i a4 = *reinterpret_cast<const v4i*>(lds + L.x0 + mc * (nblk4 * 16) + q * 64 + g * 16);
-          const v8i xf = {a4[0], a4[1], a4[2], a4[3], 0, 0, 0, 0};
 #pragma unroll
-          for (int f = 0; f < F; ++f) acc[f] = decode_mfma<kFmtE2M1>(wf[f], xf, acc[f], s_w[f], s_x);
-        } else if (seg == 1) {
-          const v2i* p = reinterpret_cast<const v2i*>(lds + L.x1 + mc * (nblk6 * 24) + q * 96 + g * 24);
-          const v2i a = p[0], b = p[1], c = p[2];
-          const v8i xf = {a[0], a[1], b[0], b[1], c[0], c[1], 0, 0};
+        for (int gi = 0; gi < G; ++gi) {
+          if (seg == 0) {
+            const v4i a4 = *reinterpret_cast<const v4i*>(lds + L.x0 + mc[gi] * (nblk4 * 16) + q * 64 + g * 16);
+            const v8i xf = {a4[0], a4[1], a4[2], a4[3], 0, 0, 0, 0};
 #pragma unroll
-          for (int f = 0; f < F; ++f) acc[f] = decode_mfma<kFmtE3M2>(wf[f], xf, acc[f], s_w[f], s_x);
-        } else {
-          const uint8_t* p = lds + L.x2 + mc * (nblk8 * 32) + q * 128 + g * 16;
-          const v4i a4 = *reinterpret_cast<const v4i*>(p), b4v = *reinterpret_cast<const v4i*>(p + 64);
-          const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4v[0], b4v[1], b4v[2], b4v[3]};
+            for (int f = 0; f < F; ++f) acc[f][gi] = decode_mfma<kFmtE2M1>(wf[f], xf, acc[f][gi], s_w[f], s_x[gi]);
+          } else if (seg == 1) {
+            const v2i* p = reinterpret_cast<const v2i*>(lds + L.x1 + mc[gi] * (nblk6 * 24) + q * 96 + g * 24);
+            const v2i a = p[0], b = p[1], c = p[2];
+            const v8i xf = {a[0], a[1], b[0], b[1], c[0], c[1], 0, 0};
 #pragma unroll
-          for (int f = 0; f < F; ++f) acc[f] = decode_mfma<kFmtE4M3>(wf[f], xf, acc[f], s_w[f], s_x);
+            for (int f = 0; f < F; ++f) acc[f][gi] = decode_mfma<kFmtE3M2>(wf[f], xf, acc[f][gi], s_w[f], s_x[gi]);
+          } else {
+            const uint8_t* p = lds + L.x2 + mc[gi] * (nblk8 * 32) + q * 128 + g * 16;
+            const v4i a4 = *reinterpret_cast<const v4i*>(p), b4v = *reinterpret_cast<const v4i*>(p + 64);
+            const v8i xf = {a4[0], a4[1], a4[2], a4[3], b4v[0], b4v[1], b4v[2], b4v[3]};
+#pragma unroll
+            for (int f = 0; f < F; ++f) acc[f][gi] = decode_mfma<kFmtE4M3>(wf[f], xf, acc[f][gi], s_w[f], s_x[gi]);
+          }
         }
       }
     }
@@ -634,15 +656,20 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
   // ---- sum the four waves' partial tiles (D^T: lane holds token lane % 16, feature slots 4 * (lane / 16) + v of a group)
   float* partial = reinterpret_cast<float*>(lds + L.partial);
 #pragma unroll
-  for (int f = 0; f < F; ++f) *reinterpret_cast<v4f*>(partial + ((wave * F + f) * 64 + lane) * 4) = acc[f];
+  for (int f = 0; f < F; ++f)
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+      *reinterpret_cast<v4f*>(partial + ((wave * (F * G) + f * G + gi) * 64 + lane) * 4) = acc[f][gi];
   __syncthreads();
 #pragma unroll
-  for (int f = 0; f < F; ++f) {
-    if ((f & 3) != wave) continue;
+  for (int fg = 0; fg < F * G; ++fg) {
+    if ((fg & 3) != wave) continue;
+    const int f = fg / G, gi = fg % G;
     v4f sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < 4; ++w) sum += *reinterpret_cast<const v4f*>(partial + ((w * F + f) * 64 + lane) * 4);
-    if (i < M) {
+    for (int w = 0; w < 4; ++w) sum += *reinterpret_cast<const v4f*>(partial + ((w * (F * G) + fg) * 64 + lane) * 4);
+    const int m = m_base + 16 * gi + i;
+    if (m < M) {
       uint16_t h[4];
 #pragma unroll
       for (int v = 0; v < 4; ++v) h[v] = __builtin_bit_cast(uint16_t, (__bf16)sum[v]);
@@ -652,14 +679,14 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           const int e = 4 * g + v, row = row0 + 32 * (e & 7) + 16 * (e >> 3);
-          if (row < N) d[(size_t)i * N + row] = h[v];
+          if (row < N) d[(size_t)m * N + row] = h[v];
         }
       } else {
         // feature slots 4 g ... 4 g + 3 of the group are four consecutive rows
         const int per_group = 32 / PB, group = blockIdx.x / per_group, c0 = (blockIdx.x % per_group) * PB;
         const int e = 16 * f + 4 * g;
         const int nn = group * 128 + c0 + e % PB + 32 * (e / PB);
-        uint16_t* dst = d + (size_t)i * N + nn;
+        uint16_t* dst = d + (size_t)m * N + nn;
         if (nn + 3 < N && (N & 3) == 0) {
           *reinterpret_cast<v2u*>(dst) = v2u{(unsigned)h[0] | ((unsigned)h[1] << 16), (unsigned)h[2] | ((unsigned)h[3] << 16)};
         } else {
@@ -674,19 +701,22 @@ mixed_gemm_decode_kernel(DecodeSeg s4, DecodeSeg s6, DecodeSeg s8, int M, int N,
 
 static int round_up_1k(int v) { return (v + 1023) & ~1023; }
 
-// The decode kernel takes: up to 16 tokens, whole 128-wide steps in every segment, and an LDS image of at most
-// 76 KB (two workgroups per CU).
-static bool decode_lds_plan(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int F, DecodeLds* L) {
+// The decode kernel takes whole 128-wide steps in every segment and, with one token group per workgroup (G = 1), up to
+// 16 tokens and an LDS image of at most 76 KB (two workgroups per CU); with two (G = 2: 32 tokens per workgroup, any
+// number of tokens below 256) whatever fits the LDS of a CU.
+constexpr int kDecodeLds1 = 76 * 1024, kDecodeLds2 = 156 * 1024;
+static bool decode_lds_plan(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int F, int G, DecodeLds* L) {
   int pos = 0;
   auto take = [&](int bytes) { const int at = pos; pos += round_up_1k(bytes); return at; };
-  L->pa = M <= 8 ? 8 : 16;
-  L->x0 = take(M * d4.nblk * 16); L->x1 = take(M * d6.nblk * 24); L->x2 = take(M * d8.nblk * 32);
+  const int rows = G == 1 ? M : (M < 32 ? M : 32);   // token rows of a workgroup's image
+  L->pa = G == 2 ? 32 : (M <= 8 ? 8 : 16);
+  L->x0 = take(rows * d4.nblk * 16); L->x1 = take(rows * d6.nblk * 24); L->x2 = take(rows * d8.nblk * 32);
   L->sfa0 = take(d4.steps * L->pa * 16); L->sfa1 = take(d6.steps * L->pa * 16); L->sfa2 = take(d8.steps * L->pa * 16);
   L->sfb0 = take(d4.steps * F * 64); L->sfb1 = take(d6.steps * F * 64); L->sfb2 = take(d8.steps * F * 64);
   L->partial = pos;
-  pos += 4 * F * 1024;
+  pos += 4 * F * G * 1024;
   L->total = pos;
-  return pos <= 76 * 1024;
+  return pos <= (G == 1 ? kDecodeLds1 : kDecodeLds2);
 }
 
 // Feature groups of 16 per workgroup of the decode kernel (and what the cost model below assumes of the skinny one).
@@ -713,6 +743,16 @@ static void skinny_groups(int rows, int N, int cus, int* g_out, int* f_out) {
   *g_out = 1;
   *f_out = 1;
 }
+// Feature groups of 16 per workgroup (4, 2 or 1) for the decode kernel with two token groups per workgroup: the most
+// that still leave most CUs a workgroup and whose LDS image fits; 0 if none does (then *L is not valid).
+static int decode2_feature_groups(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int N, int cus,
+                                  DecodeLds* L) {
+  const int tg = ceil_div(M, 32);
+  int f = ceil_div(N, 64) * tg >= cus * 3 / 4 ? 4 : (ceil_div(N, 32) * tg >= cus * 3 / 4 ? 2 : 1);
+  while (f > 1 && !decode_lds_plan(d4, d6, d8, M, f, 2, L)) f >>= 1;
+  return decode_lds_plan(d4, d6, d8, M, f, 2, L) ? f : 0;
+}
+
 hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int M, int N,
                          bool w_tiled, uint16_t* d, hipStream_t stream) {
   const int rows = M;
@@ -721,23 +761,43 @@ hipError_t launch_skinny(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeS
   // decode: the kernel that stages everything but the weight codes in LDS
   // (a segment's weight codes below 4 GB: the kernel addresses them with 32-bit per-lane offsets)
   const size_t widest = (size_t)(d4.nblk > d6.nblk ? (d4.nblk > d8.nblk ? d4.nblk : d8.nblk) : (d6.nblk > d8.nblk ? d6.nblk : d8.nblk));
-  if (M <= 16 && ((d4.nblk | d6.nblk | d8.nblk) & 3) == 0 && (size_t)N * widest * 16 < ((size_t)1 << 32)) {
+  typedef void (*kernel_t)(DecodeSeg, DecodeSeg, DecodeSeg, int, int, int, DecodeLds, uint16_t*);
+  const bool whole_steps = ((d4.nblk | d6.nblk | d8.nblk) & 3) == 0 && (size_t)N * widest * 16 < ((size_t)1 << 32);
+  const int spw = (d4.steps + d6.steps + d8.steps + 3) / 4;
+  if (M <= 16 && whole_steps) {
     // feature groups of 16 per workgroup: 4 (tile-major weights; measured on N = 14336: 9.0 against 9.6 us) or 2 as
     // long as that leaves most CUs a workgroup
     int f = skinny_feature_groups(rows, N, lim.cus);
     if (w_tiled && ceil_div(N, 64) >= lim.cus * 3 / 4) f = 4;
     DecodeLds L;
-    if (f == 4 && !decode_lds_plan(d4, d6, d8, M, f, &L)) f = 2;
-    if (decode_lds_plan(d4, d6, d8, M, f, &L)) {
-      const int spw = (d4.steps + d6.steps + d8.steps + 3) / 4;
+    if (f == 4 && !decode_lds_plan(d4, d6, d8, M, f, 1, &L)) f = 2;
+    if (decode_lds_plan(d4, d6, d8, M, f, 1, &L)) {
       // row-major: per group of 128 rows 8 / F workgroups (the last group whole, rows past N clamped and not stored)
       const dim3 grid(w_tiled ? ceil_div(N, 16 * f) : ceil_div(N, 128) * (8 / f));
-      typedef void (*kernel_t)(DecodeSeg, DecodeSeg, DecodeSeg, int, int, int, DecodeLds, uint16_t*);
       const kernel_t kernels[2][3] = {
-          {mixed_gemm_decode_kernel<1, false>, mixed_gemm_decode_kernel<2, false>, mixed_gemm_decode_kernel<4, false>},
-          {mixed_gemm_decode_kernel<1, true>, mixed_gemm_decode_kernel<2, true>, mixed_gemm_decode_kernel<4, true>}};
+          {mixed_gemm_decode_kernel<1, false, 1>, mixed_gemm_decode_kernel<2, false, 1>, mixed_gemm_decode_kernel<4, false, 1>},
+          {mixed_gemm_decode_kernel<1, true, 1>, mixed_gemm_decode_kernel<2, true, 1>, mixed_gemm_decode_kernel<4, true, 1>}};
       const kernel_t kernel = kernels[w_tiled ? 1 : 0][f == 4 ? 2 : f - 1];
-      if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), 76 * 1024); e != hipSuccess) return e;
+      if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kDecodeLds1); e != hipSuccess) return e;
+      hipLaunchKernelGGL(kernel, grid, dim3(256), (size_t)L.total, stream, d4, d6, d8, M, N, spw, L, d);
+      return hipGetLastError();
+    }
+  }
+  // More tokens, in groups of 32 per workgroup, while their codes fit the LDS (K = 4096: 79 KB; not K = 14336): the
+  // token fragments and scales then come from LDS once per workgroup instead of from memory in every K step, which
+  // is what the kernel below spends most of its time on (M = 128, N = 4096, K = 4096: 17 -> 9 us).  The most feature
+  // groups per workgroup (4, 2, 1) that still leave most CUs a workgroup.
+  if (M > 16 && whole_steps) {
+    const int tg = ceil_div(M, 32);
+    DecodeLds L;
+    const int f = decode2_feature_groups(d4, d6, d8, M, N, lim.cus, &L);
+    if (f > 0) {
+      const dim3 grid(w_tiled ? ceil_div(N, 16 * f) : ceil_div(N, 128) * (8 / f), tg);
+      const kernel_t kernels[2][3] = {
+          {mixed_gemm_decode_kernel<1, false, 2>, mixed_gemm_decode_kernel<2, false, 2>, mixed_gemm_decode_kernel<4, false, 2>},
+          {mixed_gemm_decode_kernel<1, true, 2>, mixed_gemm_decode_kernel<2, true, 2>, mixed_gemm_decode_kernel<4, true, 2>}};
+      const kernel_t kernel = kernels[w_tiled ? 1 : 0][f == 4 ? 2 : f - 1];
+      if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kDecodeLds2); e != hipSuccess) return e;
       hipLaunchKernelGGL(kernel, grid, dim3(256), (size_t)L.total, stream, d4, d6, d8, M, N, spw, L, d);
       return hipGetLastError();
     }
@@ -774,17 +834,27 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
                                  int m_store, int a_rows, int N, int KN, int KS, int KO, bool w_tiled, void* d,
                                  hipStream_t stream);
 
-// Rough launch times in microseconds, only to choose between the two kernels for fewer than 256 tokens (measured on
+// Rough launch times in microseconds, only to choose between the kernels for fewer than 256 tokens (measured on
 // MI355X, 256 CUs, K = 4096: the whole-tile kernel runs such problems as 256 x 128 tiles when that is at most one
-// round -- a 128-wide stage then takes ~0.5 us with at most half of the CUs busy, ~0.6 us with more, plus ~2.5 us --
-// and as 256 x 256 tiles at ~1.05 us a stage plus ~3 us a round otherwise; the skinny kernel takes 0.18-0.25 ns per
-// 16 tokens x 16 features x 128 K plus ~5 us).
+// round -- a 128-wide stage then takes ~0.42 us with at most half of the CUs busy, ~0.45 us with more, plus ~2.5 us --
+// and as 256 x 256 tiles at ~0.95 us a stage plus ~3 us a round otherwise; the decode kernel with two token groups
+// per workgroup takes ~5.5 us plus 22 ns per K step and feature group for each round of one workgroup per CU; the
+// skinny kernel 0.18-0.25 ns per 16 tokens x 16 features x 128 K plus ~5 us).
 static double pipelined_us(int M, int N, int stages, int cus) {
   const int whole = ceil_div(M, 256) * ceil_div(N, 256);
-  if (whole <= cus / 2) return stages * (ceil_div(M, 128) * ceil_div(N, 256) <= cus / 2 ? 0.5 : 0.6) + 2.5;
-  return (double)ceil_div(whole, cus) * (stages * 1.05 + 3.0);
+  if (whole <= cus / 2) return stages * (ceil_div(M, 128) * ceil_div(N, 256) <= cus / 2 ? 0.42 : 0.45) + 2.5;
+  return (double)ceil_div(whole, cus) * (stages * 0.95 + 3.0);
 }
-static double skinny_us(int rows, int N, int steps, int cus) {
+static double skinny_us(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSeg& d8, int rows, int N, int steps, int cus,
+                        bool w_tiled) {
+  if (rows > 16 && ((d4.nblk | d6.nblk | d8.nblk) & 3) == 0) {
+    DecodeLds L;
+    const int f2 = decode2_feature_groups(d4, d6, d8, rows, N, cus, &L);
+    if (f2 > 0) {
+      const int wgs = (w_tiled ? ceil_div(N, 16 * f2) : ceil_div(N, 128) * (8 / f2)) * ceil_div(rows, 32);
+      return 1.0 + ceil_div(wgs, cus) * (5.5 + steps * f2 * 0.022);
+    }
+  }
   int g, f;
   skinny_groups(rows, N, cus, &g, &f);
   return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * (f == 2 ? 0.18e-3 : 0.25e-3);
@@ -809,13 +879,13 @@ hipError_t launch_mixed_gemm(const uint8_t* an, const uint8_t* bn, const uint8_t
   }
   // whole 256-row tiles; the last one does not write rows past M and reads no activation row past
   // a_rows (lanes that would are pointed at the last readable row)
-  if (mixed_gemm_256_supported(m_pad, N, KN, KS, KO) &&
-      (M >= 256 || pipelined_us(M, N, steps, cus) < skinny_us(M, N, steps, cus)))
-    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, a_rows, N, KN, KS, KO,
-                                 w_tiled, d, stream);
   const DecodeSeg d4 = {an, bn, sfan, sfbn, KN / 32, (KN + 127) / 128};
   const DecodeSeg d6 = {as_, bs, sfas, sfbs, KS / 32, (KS + 127) / 128};
   const DecodeSeg d8 = {ao, bo, sfao, sfbo, KO / 32, (KO + 127) / 128};
+  if (mixed_gemm_256_supported(m_pad, N, KN, KS, KO) &&
+      (M >= 256 || pipelined_us(M, N, steps, cus) < skinny_us(d4, d6, d8, M, N, steps, cus, w_tiled)))
+    return launch_mixed_gemm_256(an, bn, as_, bs, ao, bo, sfan, sfbn, sfas, sfbs, sfao, sfbo, M, a_rows, N, KN, KS, KO,
+                                 w_tiled, d, stream);
   if (M < 256 && KN + KS + KO > 0) return launch_skinny(d4, d6, d8, M, N, w_tiled, static_cast<uint16_t*>(d), stream);
   // what is left (256 tokens or more with N not a multiple of 8, or with a segment that is not whole 128-wide
   // stages next to an empty one): the direct kernel

@@ -220,6 +220,40 @@ def test_decode_kernel_matches_oracle(abi, m, n, kn, ks, ko, tiled):
     _check_gemm(d, qx, qw, f"decode {m}x{n}x{k}")
 
 
+# 17 to 255 tokens with whole 128-wide steps: the decode kernel with two token groups (32 tokens) per workgroup where
+# the tokens' codes fit the LDS, one to four feature groups per workgroup, ragged token and feature counts, an empty
+# segment, a token count whose last workgroup has a single token group; K = 14336 does not fit (skinny kernel)
+SMALL_M_SHAPES = [
+    (128, 4096, 2560, 1408, 128), (32, 512, 2560, 1408, 128), (100, 4096, 2560, 1408, 128), (255, 512, 384, 256, 128),
+    (40, 14336, 2560, 1408, 128), (64, 256, 0, 384, 128), (130, 1000, 1280, 0, 256), (17, 264, 128, 128, 128),
+    (49, 2048, 512, 0, 0), (200, 768, 2560, 1408, 128), (33, 4096, 8960, 4928, 448),
+]
+
+
+@pytest.mark.parametrize("m,n,kn,ks,ko", SMALL_M_SHAPES)
+@pytest.mark.parametrize("tiled", [False, True])
+def test_small_batches_match_oracle(abi, m, n, kn, ks, ko, tiled):
+    k = kn + ks + ko
+    _say("small batch", m, n, kn, ks, ko, "tiled" if tiled else "row-major")
+    if tiled and not abi.weights_tileable(n, kn, ks, ko):
+        pytest.skip("shape cannot be tiled")
+    x = H.make_activations(m, k, 27 + m + n, n_out=max(1, k // 32))
+    w = H.make_weights(n, k, 29 + m + n)
+    idx = H.absmax_sort_index(x)
+    qx, qw = _oracle_operands(x, w, idx, kn, ks, ko)
+    a, b = _to_dev(qx), _to_dev(qw)
+    if tiled:
+        b = list(abi.tile_weights(*b[:3])) + b[3:]
+    d = abi.matmul(a[0], b[0], a[1], b[1], a[2], b[2], a[3], b[3], a[4], b[4], a[5], b[5], w_tiled=tiled)
+    torch.cuda.synchronize()
+    _check_gemm(d, qx, qw, f"small batch {m}x{n}x{k}")
+    # exact-size activation buffers: nothing is read past the last token's codes
+    tight = [t.clone() for t in a]
+    d2 = abi.matmul(tight[0], b[0], tight[1], b[1], tight[2], b[2], tight[3], b[3], tight[4], b[4], tight[5], b[5], w_tiled=tiled)
+    torch.cuda.synchronize()
+    assert torch.equal(d, d2)
+
+
 @pytest.mark.parametrize("m,n,kn,ks,ko", GEMM_SHAPES)
 def test_mixed_gemm_matches_oracle(abi, m, n, kn, ks, ko):
     k = kn + ks + ko

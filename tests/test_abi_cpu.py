@@ -77,7 +77,9 @@ def test_validation_of_the_newer_entry_points(abi):
     assert lib.mg_weights_tileable(4096, 8960, 4928, 448) == 1      # 32-granular segments are fine
     assert lib.mg_weights_tileable(4096, 2560, 1408, 64) == 0       # a segment narrower than one stage
     assert lib.mg_weights_tileable(1000, 2560, 1408, 128) == 0      # N not a multiple of 256
-    assert lib.mg_weights_tileable(256, 256, 0, 128) == 0           # an empty segment after fewer than three stages
+    assert lib.mg_weights_tileable(256, 256, 0, 128) == 1           # an empty segment: whole stages in the others
+    assert lib.mg_weights_tileable(256, 0, 384, 0) == 1 and lib.mg_weights_tileable(512, 0, 0, 128) == 1
+    assert lib.mg_weights_tileable(256, 416, 0, 160) == 0           # an empty segment next to segments that are not whole stages
     # plans without E3M2 and / or E4M3 activations: whole 128-wide stages, three of them before a following segment
     assert lib.mg_weights_tileable(256, 4096, 0, 0) == 1 and lib.mg_weights_tileable(256, 128, 0, 0) == 1
     assert lib.mg_weights_tileable(256, 3968, 0, 128) == 1 and lib.mg_weights_tileable(256, 2560, 1536, 0) == 1

@@ -80,10 +80,10 @@ def test_validation_of_the_newer_entry_points(abi):
     assert lib.mg_weights_tileable(256, 256, 0, 128) == 1           # an empty segment: whole stages in the others
     assert lib.mg_weights_tileable(256, 0, 384, 0) == 1 and lib.mg_weights_tileable(512, 0, 0, 128) == 1
     assert lib.mg_weights_tileable(256, 416, 0, 160) == 0           # an empty segment next to segments that are not whole stages
-    # plans without E3M2 and / or E4M3 activations: whole 128-wide stages, three of them before a following segment
+    # plans without one or two of the activation formats: whole 128-wide stages
     assert lib.mg_weights_tileable(256, 4096, 0, 0) == 1 and lib.mg_weights_tileable(256, 128, 0, 0) == 1
     assert lib.mg_weights_tileable(256, 3968, 0, 128) == 1 and lib.mg_weights_tileable(256, 2560, 1536, 0) == 1
-    assert lib.mg_weights_tileable(256, 0, 3968, 128) == 0 and lib.mg_weights_tileable(256, 4064, 0, 32) == 0
+    assert lib.mg_weights_tileable(256, 0, 3968, 128) == 1 and lib.mg_weights_tileable(256, 4064, 0, 32) == 0
     assert lib.mg_weights_tileable(256, -128, 0, 0) == 0 and lib.mg_weights_tileable(256, 512, -128, 0) == 0
     # a_rows below M, unknown flag bits, tile-major flag on a shape that cannot be tiled
     assert lib.mg_mixed_gemm_ex(*twelve, 8, 4, 256, 128, 128, 128, 0, null, null) == 10001

@@ -414,14 +414,14 @@ struct HalfFrags {
 struct WeightPtrs {
   const uint8_t* w;    // weights: row 32*t + i at block i%16, quad 8*(i/16) + t; + t*64 + h*32
   const uint8_t* sw;   // scale dwords of the 4 feature tiles
-  const uint8_t* sx;   // scale dwords of the 4 token tiles
+  const uint8_t* sx;   // scale dwords of the wave's token tiles
 
   // the wave's token tiles lie in scale atom c.xatom of the workgroup's tile
   __device__ __forceinline__ WeightPtrs(const uint8_t* lds, const Ctx& c) {
     const int i = c.lane & 31, g = c.lane >> 5;
     w = lds + kWOff + (i & 15) * kBlk + (i >> 4) * 512 + c.wn * 256 + g * 16;
     sw = lds + kSOff + c.wn * 512 + i * 16;
-    sx = lds + kSOff + 1024 + c.xatom * 512 + i * 16;
+    sx = lds + kSOff + 1024 + c.xatom * 512 + i * 16 + c.xtile * 4;
   }
 };
 
@@ -479,7 +479,14 @@ struct FragReader {
     } else if constexpr (SC && R == 4 + TM) {
       sw = *reinterpret_cast<const v4i*>(psw);
     } else if constexpr (SC && R == 5 + TM) {
-      sx = *reinterpret_cast<const v4i*>(psx);
+      // the dwords of the wave's own token tiles only (TM consecutive ones of the atom's four)
+      if constexpr (TM == 2) {
+        const v2i t = *reinterpret_cast<const v2i*>(psx);
+        sx[0] = t[0];
+        sx[1] = t[1];
+      } else {
+        sx[0] = *reinterpret_cast<const int*>(psx);
+      }
     }
   }
 };
@@ -492,24 +499,28 @@ __device__ __forceinline__ void read_all(const FragReader<FMT, H, SC, TM>& rd) {
   }
 }
 
+// reads [R0, R1) of a half's fragments, as far as there are that many
+template <int R0, int R1, class Reader>
+__device__ __forceinline__ void read_some(const Reader& rd) {
+  if constexpr (R0 < R1 && R0 < Reader::kReads) {
+    rd.template read<R0>();
+    read_some<R0 + 1, R1>(rd);
+  }
+}
+
 template <int TM>
 struct Scales {
   int w[4], x[TM];   // scale dwords of the 4 feature / TM token tiles, shifted so that byte 0 / 2 is block g / 2+g
 };
 
-// sx holds the dwords of the four token tiles of a scale atom; the wave's are xtile ... xtile + TM - 1 (xtile wave-uniform)
+// sw holds the scale dwords of the four feature tiles, sx[0 .. TM - 1] those of the wave's token tiles
 template <int TM>
-__device__ __forceinline__ void shift_scales(Scales<TM>& sc, v4i sw, v4i sx, int lane, int xtile) {
+__device__ __forceinline__ void shift_scales(Scales<TM>& sc, v4i sw, v4i sx, int lane) {
   const int g8 = (lane >> 5) * 8;
 #pragma unroll
   for (int t = 0; t < 4; ++t) sc.w[t] = (int)((unsigned)sw[t] >> g8);
 #pragma unroll
-  for (int t = 0; t < TM; ++t) {
-    int v;
-    if constexpr (TM == 2) v = xtile ? sx[2 + t] : sx[t];
-    else v = xtile == 0 ? sx[0] : (xtile == 1 ? sx[1] : (xtile == 2 ? sx[2] : sx[3]));
-    sc.x[t] = (int)((unsigned)v >> g8);
-  }
+  for (int t = 0; t < TM; ++t) sc.x[t] = (int)((unsigned)sx[t] >> g8);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -539,11 +550,10 @@ __device__ __forceinline__ void mfma_half(v16f (&acc)[4][TM], const HalfFrags<FM
   if constexpr (M0 < 4 * TM) {
     constexpr int tn = M0 / TM, tm = M0 % TM;
     mfma_one<FMT, H>(acc[tn][tm], f.w[tn], f.x[tm], sc.w[tn], sc.x[tm]);
-    // one fragment read per MFMA, two where a half has fewer MFMAs than reads (TM == 1)
-    constexpr int RP = (Reader::kReads + 4 * TM - 1) / (4 * TM);
-    if constexpr (M0 * RP < Reader::kReads) rd.template read<M0 * RP>();
-    if constexpr (RP == 2 && M0 * RP + 1 < Reader::kReads) rd.template read<M0 * RP + 1>();
-    static_assert(RP <= 2, "fragment reads per MFMA");
+    // The fragment reads go out after the first MFMAs, as few per MFMA as leaves the last two MFMAs of the half
+    // without one: what is read last is needed first afterwards, and its LDS latency would stand between two halves.
+    constexpr int RP = (Reader::kReads + 4 * TM - 3) / (4 * TM - 2);
+    read_some<M0 * RP, (M0 + 1) * RP>(rd);
     constexpr int KS = LEAN ? (CF == kFmtNone ? K1 : next_slot<CF>(K0)) : K0;
     // a copy slot after every second MFMA where a wave has twice as many MFMAs per half as copy slots, else after every one
     constexpr bool kEvery = 4 * TM <= kCopySlots - kSplit;
@@ -619,7 +629,7 @@ __device__ __forceinline__ void stage_body(v16f (&acc)[4][TM], HalfFrags<FMT, TM
   mfma_half<FMT, 1, LEAN, CE, 0, 0, kSplit>(acc, b, sc, rd_n, lce, early_on, ring.cur, gc, lo, c.wave);
   __builtin_amdgcn_sched_barrier(0);
   wait_lds_reads();
-  shift_scales(sc, sw, sx, c.lane, c.xtile);
+  shift_scales(sc, sw, sx, c.lane);
   if constexpr (FR == FMT) a = nx;
   else a_next = nx;
 }
@@ -1008,7 +1018,7 @@ __device__ __forceinline__ void compute_tile(const Plan& plan, int tile_n, int t
     const FragReader<FA, 0, true, TM> rd{fa, sw, sx, wp.w, xp.x, wp.sw, wp.sx, true};
     read_all(rd);
     wait_lds_reads();
-    shift_scales(sc, sw, sx, c.lane, c.xtile);
+    shift_scales(sc, sw, sx, c.lane);
   }
   LeanCopy<kFmtNone, WT> l0;
   // NLAST goes to the plan's last segment and the one before it (see run_segment)

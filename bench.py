@@ -158,6 +158,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--no-zero-operand-leg", action="store_true",
+                    help="skip the c3 launches on all-zero operand codes (same kernel and grid as c3: in a kernel trace "
+                         "they would be averaged into c3's row)")
     ap.add_argument("--no-clock-warmup", action="store_true",
                     help="skip the 0.4 s of untimed steps in front (for counter runs, where every launch is slow)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -321,21 +324,22 @@ def main():
         # ------------------------------------------------------------ the same launch on all-zero operands: same
         # instructions, addresses and bytes moved, but the multiplier arrays do not toggle -- separates what the
         # kernel's structure costs from what the chip's power limit costs on real operand bits
-        zq = abi.reorder_quantize_x(torch.zeros_like(xd), idd, kn, ks, ko)
-        zw = abi.reorder_quantize_w(torch.zeros_like(wd), idd, kn, ks, ko)
-        zb = abi.tile_weights(*zw[:3])
-        zr, rr = [], []
-        for _ in range(5):   # straight after the leg above: the GPU has not idled
-            zr.append(graph_ms(lambda i: abi.matmul(zq[0], zb[0], zq[1], zb[1], zq[2], zb[2], zq[3], zw[3], zq[4], zw[4],
-                                                    zq[5], zw[5], out=d, w_tiled=True), 20, repeats=2, warm_s=0.0))
-            rr.append(graph_ms(lambda i: abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4],
-                                                    aq[5], bq[5], out=d, w_tiled=True), 20, repeats=2, warm_s=0.0))
-        z_ms, r_ms = sorted(zr)[2], sorted(rr)[2]
-        extra["gemm_c3_zero_operands"] = {
-            "note": "c3 GEMM launch with all-zero operand codes against the bench operands, medians of 5 interleaved runs of 20 launches",
-            "zero_ms": round(z_ms, 5), "zero_tflops": round(flops / (z_ms * 1e-3) / 1e12, 1),
-            "bench_operands_ms": round(r_ms, 5), "bench_operands_tflops": round(flops / (r_ms * 1e-3) / 1e12, 1)}
-        del zq, zw, zb
+        if not args.no_zero_operand_leg:
+            zq = abi.reorder_quantize_x(torch.zeros_like(xd), idd, kn, ks, ko)
+            zw = abi.reorder_quantize_w(torch.zeros_like(wd), idd, kn, ks, ko)
+            zb = abi.tile_weights(*zw[:3])
+            zr, rr = [], []
+            for _ in range(5):   # straight after the leg above: the GPU has not idled
+                zr.append(graph_ms(lambda i: abi.matmul(zq[0], zb[0], zq[1], zb[1], zq[2], zb[2], zq[3], zw[3], zq[4], zw[4],
+                                                        zq[5], zw[5], out=d, w_tiled=True), 20, repeats=2, warm_s=0.0))
+                rr.append(graph_ms(lambda i: abi.matmul(aq[0], bt[0], aq[1], bt[1], aq[2], bt[2], aq[3], bq[3], aq[4], bq[4],
+                                                        aq[5], bq[5], out=d, w_tiled=True), 20, repeats=2, warm_s=0.0))
+            z_ms, r_ms = sorted(zr)[2], sorted(rr)[2]
+            extra["gemm_c3_zero_operands"] = {
+                "note": "c3 GEMM launch with all-zero operand codes against the bench operands, medians of 5 interleaved runs of 20 launches",
+                "zero_ms": round(z_ms, 5), "zero_tflops": round(flops / (z_ms * 1e-3) / 1e12, 1),
+                "bench_operands_ms": round(r_ms, 5), "bench_operands_tflops": round(flops / (r_ms * 1e-3) / 1e12, 1)}
+            del zq, zw, zb
         # ------------------------------------------------------------ the weight side of the reorder-quantize kernel
         # (run_reorder_bf16_fp4, timed by bench_reorder.cu:143-166 of the reference next to the activation side):
         # c3's W[14336, 4096] -> three E2M1 segments + scales, then the tile-major rewrite of the codes; offline work
@@ -518,10 +522,11 @@ def main():
                                          "Infinity Cache); 20 launches per kernel replayed as a HIP graph: 0.15 s of untimed replays, then the median of 5", "rows": matrix}
 
         # ------------------------------------------------------------ one activation format at a time (c3's M, N, K)
-        # splits that run the kernels c3 runs (segment-boundary copies compiled in: at least three stages in each of
-        # the first two segments), tile-major weights; the other two formats get the fewest stages that allows
+        # splits that run the kernel family c3 runs (segment-boundary copies compiled in: at least three stages in every
+        # segment that another follows), tile-major weights; the other formats get few stages, and the last segments
+        # differ in length (2, 3 stages; no E3M2 at all) so that each leg is a kernel of its own in a trace
         per_format = []
-        for name, (knf, ksf, kof) in (("e2m1", (3584, 384, 128)), ("e3m2", (384, 3584, 128)), ("e4m3", (384, 384, 3328))):
+        for name, (knf, ksf, kof) in (("e2m1", (3456, 384, 256)), ("e3m2", (384, 3328, 384)), ("e4m3", (768, 0, 3328))):
             aqf = abi.reorder_quantize_x(xd, idd, knf, ksf, kof)
             wqf = abi.reorder_quantize_w(wd, idd, knf, ksf, kof)
             wqf = abi.tile_weights(*wqf[:3]) + wqf[3:]
@@ -533,8 +538,8 @@ def main():
             per_format.append({"activations": name, "split": [knf, ksf, kof], "gemm_ms": round(f_ms, 5),
                                "tflops": round(tf, 1), "peak": round(pk, 1), "frac": round(tf / pk, 4)})
             del aqf, wqf, df
-        extra["per_format_gemm"] = {"note": "c3's M, N and K with 3584 (E4M3: 3328) of the 4096 channels in one activation format, "
-                                            "on the kernels c3 runs; peak = the same blended nominal formula", "rows": per_format}
+        extra["per_format_gemm"] = {"note": "c3's M, N and K with 3456 / 3328 / 3328 of the 4096 channels in one activation format, "
+                                            "on the kernel family c3 runs; peak = the same blended nominal formula", "rows": per_format}
 
         # ------------------------------------------------------------ plans without one or two of the activation formats
         # (the last three: pure E3M2 x E2M1 and E4M3 x E2M1 products, what matmul_host6 / matmul_host8 of the

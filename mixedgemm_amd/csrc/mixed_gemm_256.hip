@@ -1257,16 +1257,28 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
 __global__ void __launch_bounds__(256) tile_weights_kernel(const v4u* __restrict__ src, v4u* __restrict__ dst, int N, int blk) {
   const int nst = blk >> 2, rem = blk & 3;
   const size_t tiled = (size_t)N * nst * 4;   // 16-byte units in whole stages
-  const size_t total = (size_t)N * blk;
-  for (size_t u = (size_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (size_t)gridDim.x * 256) {
-    if (u < tiled) {
-      const unsigned c = u & 3, k = (u >> 2) & 15, j = (u >> 6) & 15;
-      const size_t ts = u >> 10;   // tile_n * nst + stage
-      const unsigned ql = ts % nst;
-      const size_t tile_n = ts / nst;
+  // Whole stages: 128 lanes move the 1 KB copy block j of two neighbouring stages (lane = 8 * quad + 4 * stage parity +
+  // piece), so that the eight lanes of a quad read 128 consecutive bytes of one row -- a whole cache line -- and a wave
+  // writes 512 consecutive bytes of each of the two stages.
+  const int npairs = (nst + 1) >> 1;
+  const size_t groups = (size_t)(N >> 8) * npairs * 16;
+  const int t7 = threadIdx.x & 127;
+  const unsigned c = t7 & 3, sp = (t7 >> 2) & 1, k = t7 >> 3;
+  for (size_t g = (size_t)blockIdx.x * 2 + (threadIdx.x >> 7); g < groups; g += (size_t)gridDim.x * 2) {
+    const unsigned j = g & 15;
+    const size_t tp = g >> 4;
+    const unsigned pair = tp % npairs;
+    const size_t tile_n = tp / npairs;
+    const unsigned ql = 2 * pair + sp;
+    if (ql < (unsigned)nst) {
       const size_t row = tile_n * 256 + j + 16 * (2 * (k & 7) + (k >> 3));
-      dst[u] = src[row * blk + ql * 4 + c];
-    } else {
+      dst[(((tile_n * nst + ql) * 16 + j) << 6) + k * 4 + c] = src[row * blk + ql * 4 + c];
+    }
+  }
+  // the 1-3 blocks past the last whole stage: N row-major rows behind the tiled part
+  if (rem) {
+    const size_t total = (size_t)N * blk;
+    for (size_t u = tiled + (size_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (size_t)gridDim.x * 256) {
       const size_t v = u - tiled;
       dst[u] = src[(v / rem) * blk + nst * 4 + v % rem];
     }
@@ -1277,7 +1289,7 @@ hipError_t launch_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg
   if (N % 256 != 0 || kseg % 32 != 0) return hipErrorInvalidValue;
   if (N == 0 || kseg == 0) return hipSuccess;
   const size_t units = (size_t)N * (kseg / 32);
-  const int grid = (int)((units + 255) / 256 < 4096 ? (units + 255) / 256 : 4096);
+  const int grid = (int)((units + 255) / 256 < 8192 ? (units + 255) / 256 : 8192);
   hipLaunchKernelGGL(tile_weights_kernel, dim3(grid), dim3(256), 0, stream, reinterpret_cast<const v4u*>(src),
                      reinterpret_cast<v4u*>(dst), N, kseg / 32);
   return hipGetLastError();

@@ -117,8 +117,9 @@ int mg_mixed_gemm_ex(const uint8_t* an, const uint8_t* bn, const uint8_t* as_, c
  * N a multiple of 256, kseg a multiple of 32.  Done once per layer, offline. */
 int mg_tile_weights(const uint8_t* src, uint8_t* dst, int N, int kseg, void* stream);
 /* 1 when weights of this shape can be tiled (the shapes the whole-tile kernel takes, whole tiles only): N a multiple of
- * 256 and either every segment a multiple of 32 and at least 128 wide, or KS and / or KO zero with the
- * other segments multiples of 128 (KN >= 384 when a segment follows it). */
+ * 256 and either every segment a multiple of 32 and at least 128 wide, or one or two of the segments empty and
+ * the others multiples of 128 (pure E3M2 x E2M1 and E4M3 x E2M1 products among them: what matmul_host6 and
+ * matmul_host8 of the reference, src/fp6.cu:35 and src/fp8.cu:35, compute on their own). */
 int mg_weights_tileable(int N, int KN, int KS, int KO);
 /* M rounded up to whole 256-token tiles. */
 int mg_padded_rows(int M);

@@ -160,7 +160,7 @@ GEMM_SHAPES = [
     (20, 64, 448, 224, 64), (1, 16, 32, 32, 32),
     # decode kernel (M <= 16): ragged N, partial K steps, more K steps than one pass keeps in flight
     (8, 200, 96, 160, 64), (3, 1000, 2560, 1408, 128), (16, 48, 8192, 4096, 1024), (5, 40, 0, 4928, 448),
-    # 128 tokens x 256 features and whole 128-wide K stages (the skinny kernel, or 256 x 128 tiles where they are estimated faster)
+    # 128 tokens x 256 features and whole 128-wide K stages (the decode kernel with two token groups per workgroup, or 256 x 128 tiles where they are estimated faster)
     (128, 256, 256, 0, 0), (128, 256, 0, 256, 0), (128, 256, 0, 0, 128), (128, 256, 128, 0, 128),
     (256, 512, 384, 256, 128), (128, 256, 2560, 1408, 128), (384, 768, 1280, 640, 128),
     # whole tiles with all three segments: the one-workgroup-per-CU kernel
@@ -169,7 +169,7 @@ GEMM_SHAPES = [
     (256, 256, 384, 384, 384), (512, 256, 512, 384, 128), (256, 512, 384, 512, 256),
     # segments that end 32, 64 or 96 elements past their last whole 128-wide stage
     (256, 256, 448, 416, 224), (256, 512, 2240, 1248, 448), (512, 256, 160, 480, 352),
-    # skinny kernel with 2, 4 and 8 token groups: ragged M and N, partial K steps, an empty segment
+    # 17 to 255 tokens: ragged M and N, partial K steps (skinny kernel), an empty segment
     (17, 48, 256, 128, 128), (32, 200, 96, 160, 64), (50, 40, 2560, 1408, 128), (64, 64, 0, 4928, 448),
     (100, 256, 448, 224, 64), (128, 4096, 2560, 1408, 128), (255, 272, 128, 128, 128), (200, 1000, 640, 256, 256),
     # ragged token counts: the last 256-row tile stores only part of its rows

@@ -827,10 +827,12 @@ __device__ __forceinline__ void remainder_mfma(v16f (&acc)[4][TM], RemainderHalf
 // feature tiles and walk it feature tile by feature tile inside groups of at most 8 feature tiles, token tile
 // after token tile: the ~32 tiles an XCD works on at a time are then about as many feature tiles as token tiles
 // (7 x 4.6 for 56 x 16 tiles), which is what keeps the bytes that pass its L2 lowest.
-__device__ __forceinline__ void tile_of(int wg, int nwg, int tiles_n, int& tile_n, int& tile_m) {
+// Returns whether the banded walk applies (tile counts that divide accordingly).
+__device__ __forceinline__ bool tile_of(int wg, int nwg, int tiles_n, int& tile_n, int& tile_m) {
   const int tiles_m = nwg / tiles_n;
   tile_n = wg / tiles_m;
   tile_m = wg % tiles_m;
+  bool banded = false;
   if ((nwg & 7) == 0) {
     const int per_xcd = nwg >> 3;
     const int j = wg >> 3;                       // position in this XCD's list
@@ -845,9 +847,11 @@ __device__ __forceinline__ void tile_of(int wg, int nwg, int tiles_n, int& tile_
         const int g = j / per_group, r = j % per_group;
         tile_n = (wg & 7) * cols + g * gw + r % gw;
         tile_m = r / gw;
+        banded = true;
       }
     }
   }
+  return banded;
 }
 
 // What a workgroup does before its tile: the staggered start and the plan into scalar registers.
@@ -1115,9 +1119,20 @@ mixed_gemm_256_tail_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a
     tile_of(wg, ntiles, tiles_n, tile_n, tile_m);
     compute_tile<true, REM, WT, 7, 2, NLAST>(plan, tile_n, tile_m, tiles_n, N, m_store, a_rows, d, lds);
   } else {
-    const int h = wg - n_whole;
-    tile_of(n_whole + (h >> 1), ntiles, tiles_n, tile_n, tile_m);
-    const int half_m = 2 * tile_m + (h & 1);
+    // Where the XCDs walk bands of feature tiles, the two halves of a tile go to the XCD that holds the tile's band
+    // (workgroups 8 apart): its L2 then fetches the weight tile once for both, and the tiles left over in a band
+    // share their token rows (M = 4096, N = 14336: 250 -> 226 MB past the L2s).  Elsewhere the halves of a tile are
+    // neighbouring workgroups: an XCD then holds upper or lower halves only, of two XCDs' leftovers, which for the
+    // feature-major walk are the same token tiles (M = 4096, N = 5120, K = 13824: 443 MB that way, 502 MB paired).
+    const int h = wg - n_whole, nh = (int)gridDim.x - n_whole;
+    int t = ((h >> 4) << 3) | (h & 7), upper = (h >> 3) & 1;
+    const bool paired = tile_of(n_whole + t, ntiles, tiles_n, tile_n, tile_m) && (n_whole & 7) == 0 && (nh & 15) == 0;
+    if (!paired) {
+      t = h >> 1;
+      upper = h & 1;
+      tile_of(n_whole + t, ntiles, tiles_n, tile_n, tile_m);
+    }
+    const int half_m = 2 * tile_m + upper;
     if (half_m * 128 >= m_store) return;   // the lower half of a ragged last tile: no token of it exists
     compute_tile<true, REM, WT, 7, 1, NLAST>(plan, tile_n, half_m, tiles_n, N, m_store, a_rows, d, lds);
   }

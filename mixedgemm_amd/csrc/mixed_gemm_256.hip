@@ -827,12 +827,40 @@ __device__ __forceinline__ void remainder_mfma(v16f (&acc)[4][TM], RemainderHalf
 // feature tiles and walk it feature tile by feature tile inside groups of at most 8 feature tiles, token tile
 // after token tile: the ~32 tiles an XCD works on at a time are then about as many feature tiles as token tiles
 // (7 x 4.6 for 56 x 16 tiles), which is what keeps the bytes that pass its L2 lowest.
+// A launch of at most one tile per CU (cus > 0 says so: all its tiles run at once) gives each XCD a rectangle of
+// bn x bm tiles instead, the one of the 8 / 4 / 2 / 1 column splits that needs the fewest operand bytes per stage
+// (a weight tile is 16 KB per stage, a token tile of `tokens` rows about 80 bytes per row): M = 2048, N = 4096 as
+// 256 tiles of 256 x 128 fetches 140 MB past the L2s as 4 x 8 rectangles, 186 MB as 2 x 16 bands.
 // Returns whether the banded walk applies (tile counts that divide accordingly).
-__device__ __forceinline__ bool tile_of(int wg, int nwg, int tiles_n, int& tile_n, int& tile_m) {
+__device__ __forceinline__ bool tile_of(int wg, int nwg, int tiles_n, int& tile_n, int& tile_m, int cus = 0, int tokens = kT) {
   const int tiles_m = nwg / tiles_n;
   tile_n = wg / tiles_m;
   tile_m = wg % tiles_m;
   bool banded = false;
+  if ((nwg & 7) == 0 && nwg <= cus) {
+    // (a rectangle must beat what the walk below gives an XCD: its tiles in feature-major order, i.e. all token tiles of
+    // one or two feature tiles, and of a third where the XCDs' shares do not end with a column)
+    const int share = nwg >> 3;
+    int best = 0, best_cost = ((share + tiles_m - 1) / tiles_m + (share % tiles_m != 0 ? 1 : 0)) * 16384 +
+                              min(tiles_m, share) * tokens * 80;
+#pragma unroll
+    for (int gx = 8; gx >= 1; gx >>= 1) {
+      const int gy = 8 / gx;
+      if (tiles_n % gx == 0 && tiles_m % gy == 0) {
+        const int cost = (tiles_n / gx) * 16384 + (tiles_m / gy) * tokens * 80;
+        if (cost < best_cost) {
+          best_cost = cost;
+          best = gx;
+        }
+      }
+    }
+    if (best > 0) {
+      const int xcd = wg & 7, j = wg >> 3, bn = tiles_n / best, bm = tiles_m / (8 / best);
+      tile_n = (xcd % best) * bn + j % bn;
+      tile_m = (xcd / best) * bm + j / bn;
+      return false;
+    }
+  }
   if ((nwg & 7) == 0) {
     const int per_xcd = nwg >> 3;
     const int j = wg >> 3;                       // position in this XCD's list
@@ -1097,7 +1125,7 @@ mixed_gemm_256_kernel(Plan plan_arg, int tiles_n, int N, int m_store, int a_rows
   extern __shared__ __align__(16) uint8_t lds[];
   const Plan plan = start_workgroup<WT>(plan_arg, first_round, skew);
   int tile_n, tile_m;
-  tile_of(blockIdx.x, gridDim.x, tiles_n, tile_n, tile_m);
+  tile_of(blockIdx.x, gridDim.x, tiles_n, tile_n, tile_m, first_round, 128 * TM);
   compute_tile<REGULAR, REM, WT, SEGS, TM, NLAST>(plan, tile_n, tile_m, tiles_n, N, m_store, a_rows, d, lds);
 }
 

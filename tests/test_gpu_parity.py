@@ -285,6 +285,9 @@ BIG_TILE_SHAPES = [
     # last tile has no lower half; features that are not whole tiles)
     (4352, 4096, 384, 384, 128), (4352, 4096, 384, 384, 256), (4352, 4096, 384, 384, 384), (4352, 4096, 448, 416, 224),
     (4200, 4096, 384, 384, 128), (4300, 4104, 448, 416, 224),
+    # launches of at most one tile per CU whose tile counts divide among the 8 XCDs as rectangles of tiles
+    # (8 x 8, 16 x 12 and 8 x 16 tiles of 256 x 128; 16 x 8 tiles of 256 x 256), ragged tokens among them
+    (1024, 2048, 384, 384, 128), (1536, 4096, 384, 384, 256), (2000, 2048, 384, 128, 0), (2048, 4096, 256, 128, 128),
 ]
 
 

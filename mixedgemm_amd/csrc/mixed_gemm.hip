@@ -855,7 +855,7 @@ hipError_t launch_mixed_gemm_256(const uint8_t* an, const uint8_t* bn, const uin
 // round -- a 128-wide stage then takes ~0.42 us with at most half of the CUs busy, ~0.45 us with more, plus ~2.5 us --
 // and as 256 x 256 tiles at ~0.95 us a stage plus ~3 us a round otherwise; the decode kernel with two token groups
 // per workgroup takes ~5.5 us plus 22 ns per K step and feature group for each round of one workgroup per CU; the
-// skinny kernel 0.18-0.25 ns per 16 tokens x 16 features x 128 K plus ~5 us).
+// skinny kernel 0.25-0.33 ns per 16 tokens x 16 features x 128 K plus ~5 us: K = 14336, N = 4096, 64 / 128 tokens 28 / 62 us).
 static double pipelined_us(int M, int N, int stages, int cus) {
   const int whole = ceil_div(M, 256) * ceil_div(N, 256);
   if (whole <= cus / 2) return stages * (ceil_div(M, 128) * ceil_div(N, 256) <= cus / 2 ? 0.42 : 0.45) + 2.5;
@@ -873,7 +873,7 @@ static double skinny_us(const DecodeSeg& d4, const DecodeSeg& d6, const DecodeSe
   }
   int g, f;
   skinny_groups(rows, N, cus, &g, &f);
-  return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * (f == 2 ? 0.18e-3 : 0.25e-3);
+  return 5.0 + (double)ceil_div(rows, 16) * ceil_div(N, 16) * steps * (f == 2 ? 0.25e-3 : 0.33e-3);
 }
 
 // a_rows: token rows for which the activation codes and scales are readable (>= M)

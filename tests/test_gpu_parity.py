@@ -198,6 +198,10 @@ DECODE_SHAPES = [
     (2, 9000, 4096, 2048, 512), (16, 8192, 128, 0, 0),
     # wide tile-major layers: four feature groups per workgroup; 16 tokens, and K beyond the first two rounds
     (16, 12288, 384, 256, 128), (5, 14336, 8960, 4928, 448),
+    # a last K step of 1, 2, 3 blocks of 32 in every segment; segments shorter than a step; long K whose LDS image
+    # needs a CU's whole LDS (and fewer feature groups per workgroup for 16 tokens)
+    (8, 512, 416, 480, 160), (16, 768, 160, 224, 352), (4, 1024, 480, 448, 192), (9, 520, 64, 96, 32),
+    (8, 4096, 8960, 4928, 448), (16, 4096, 7680, 4224, 384), (1, 3584, 11776, 6560, 608),
 ]
 
 
@@ -227,6 +231,7 @@ SMALL_M_SHAPES = [
     (128, 4096, 2560, 1408, 128), (32, 512, 2560, 1408, 128), (100, 4096, 2560, 1408, 128), (255, 512, 384, 256, 128),
     (40, 14336, 2560, 1408, 128), (64, 256, 0, 384, 128), (130, 1000, 1280, 0, 256), (17, 264, 128, 128, 128),
     (49, 2048, 512, 0, 0), (200, 768, 2560, 1408, 128), (33, 4096, 8960, 4928, 448),
+    (32, 512, 416, 480, 160), (64, 1024, 160, 224, 352), (100, 768, 480, 448, 192),
 ]
 
 
